@@ -1,0 +1,109 @@
+/*
+ * mfq -- group-wise affine quantization and quantized matmul for one
+ * MI355X (gfx950).  C ABI of libmfq.so.
+ *
+ * This is the boundary a host runtime binds to replace the three MLX
+ * operations mflux's quantized-linear path lands in.  mflux has no FFI of its
+ * own for this path: it calls mlx.nn.quantize and then invokes the resulting
+ * QuantizedLinear modules, so each entry point below cites the reference call
+ * site(s) whose work it performs.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer on the current HIP device, row-major
+ *     and densely packed; the caller owns all buffers;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     all calls are asynchronous on it and perform no allocation other than
+ *     where stated;
+ *   - dtype codes are MFQ_F32 / MFQ_F16 / MFQ_BF16;
+ *   - the return value is MFQ_OK (0) or a negative MFQ_E* code; nothing is
+ *     thrown across the boundary and nothing is launched when an error is
+ *     returned.  mfq_strerror() names a code.
+ *   - packed layout (identical to MLX's): element i of a row is the
+ *     `bits`-wide field at bit offset (i % (32/bits)) * bits of the uint32
+ *     word i / (32/bits); scales and biases hold one value per `group_size`
+ *     consecutive elements of a row.
+ */
+#ifndef MFQ_H
+#define MFQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum mfq_dtype { MFQ_F32 = 0, MFQ_F16 = 1, MFQ_BF16 = 2 };
+
+enum mfq_status {
+  MFQ_OK = 0,
+  MFQ_EDTYPE = -1,     /* unknown or unsupported dtype code                  */
+  MFQ_EGROUP = -2,     /* group_size not in {32, 64, 128}                    */
+  MFQ_EBITS = -3,      /* bits not in {4, 8}                                 */
+  MFQ_ESHAPE = -4,     /* K not a multiple of group_size, or a size <= 0     */
+  MFQ_ENULL = -5,      /* a required pointer is NULL                         */
+  MFQ_EALIGN = -6,     /* a buffer is not 16-byte aligned                    */
+  MFQ_ELAUNCH = -7,    /* the HIP runtime refused the launch                 */
+  MFQ_EUNSUPPORTED = -8 /* valid request that this build has no kernel for   */
+};
+
+/* Library version: major*10000 + minor*100 + patch. */
+int mfq_version(void);
+
+/* Static, never-NULL description of a status code. */
+const char* mfq_strerror(int status);
+
+/*
+ * Quantize `rows` rows of K elements each.
+ * Replaces mx.quantize(w, group_size, bits, mode="affine") as reached from
+ * nn.quantize at src/mflux/models/common/weights/loading/
+ * weight_applier.py:43,46,103 (Linear.to_quantized -> QuantizedLinear.
+ * from_linear).  Results are bit-identical to MLX's CPU evaluation.
+ *   w       [rows, K]              dtype
+ *   wq      [rows, K*bits/32]      uint32
+ *   scales  [rows, K/group_size]   dtype
+ *   biases  [rows, K/group_size]   dtype
+ */
+int mfq_quantize_affine(const void* w, int dtype, int64_t rows, int64_t K,
+                        int group_size, int bits, uint32_t* wq, void* scales,
+                        void* biases, void* stream);
+
+/*
+ * Inverse mapping w = code*scale + bias, written in `out_dtype`.
+ * Replaces mx.dequantize; mflux needs it where a LoRA is baked into a
+ * quantized base (src/mflux/models/common/lora/mapping/lora_saver.py:59-82).
+ * The value is the float32 fma(code, scale, bias) rounded once to out_dtype.
+ */
+int mfq_dequantize_affine(const uint32_t* wq, const void* scales,
+                          const void* biases, int sb_dtype, int64_t rows,
+                          int64_t K, int group_size, int bits, void* out,
+                          int out_dtype, void* stream);
+
+/*
+ * y[m, n] = sum_k x[m, k] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs])
+ *           (+ bias[n], added after y has been rounded to y_dtype, which is
+ *           what QuantizedLinear.__call__ does with its second op).
+ * Replaces mx.quantized_matmul(x, w, scales, biases, transpose=True, ...) plus
+ * the bias add of every quantized nn.Linear call, e.g.
+ *   src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53,57
+ *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12
+ *   src/mflux/models/z_image/model/z_image_transformer/feed_forward.py:13
+ *   src/mflux/models/qwen/model/qwen_transformer/qwen_transformer_block.py:36-37
+ *   x       [M, K]                 x_dtype (MFQ_BF16 or MFQ_F16; must equal sb_dtype)
+ *   wq      [N, K*bits/32]         uint32
+ *   scales  [N, K/group_size]      sb_dtype
+ *   biases  [N, K/group_size]      sb_dtype
+ *   bias    [N] or NULL            sb_dtype
+ *   y       [M, N]                 y_dtype (sb_dtype or MFQ_F32)
+ * M <= 16 runs the HBM-bound dequant-GEMV kernel, larger M the MFMA GEMM.
+ * Accumulation is float32 throughout.
+ */
+int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
+              const uint32_t* wq, const void* scales, const void* biases,
+              int sb_dtype, const void* bias, int64_t N, int group_size,
+              int bits, void* y, int y_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MFQ_H */

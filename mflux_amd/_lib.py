@@ -1,0 +1,57 @@
+"""ctypes binding of libmfq.so (the C ABI declared in include/mfq.h).
+
+There is no fallback: if the library has not been built, or a call returns an
+error code, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmfq.so")
+
+F32, F16, BF16 = 0, 1, 2
+
+# every symbol include/mfq.h declares, with its ctypes signature
+_I64, _INT, _PTR = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
+SIGNATURES = {
+    "mfq_version": (_INT, []),
+    "mfq_strerror": (ctypes.c_char_p, [_INT]),
+    "mfq_quantize_affine": (_INT, [_PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR]),
+    "mfq_dequantize_affine": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmm_t": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+}
+
+_lib = None
+
+
+class MfqError(RuntimeError):
+    """A libmfq entry point returned a negative status."""
+
+    def __init__(self, fn: str, status: int, message: str):
+        super().__init__(f"{fn} failed: {message} (status {status})")
+        self.status = status
+
+
+def load() -> ctypes.CDLL:
+    """Loads libmfq.so from the source tree; raises if it is not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -m mflux_amd._build` "
+                "(there is no CPU or PyTorch fallback for the quantized kernels)"
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+def check(fn: str, status: int) -> None:
+    if status != 0:
+        raise MfqError(fn, status, load().mfq_strerror(status).decode())

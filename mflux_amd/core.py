@@ -1,0 +1,195 @@
+"""Functional API: ``quantize``, ``dequantize``, ``quantized_matmul``.
+
+Same names, argument meaning and error behaviour as ``mx.quantize``,
+``mx.dequantize`` and ``mx.quantized_matmul`` (mode ``"affine"``), which is
+where mflux's quantized linears land: ``nn.quantize`` at
+src/mflux/models/common/weights/loading/weight_applier.py:43,46,103 and every
+quantized ``nn.Linear`` call such as
+src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53,57.
+
+Tensors are torch tensors on a HIP device; torch only provides the device
+memory and the stream, the arithmetic is libmfq's hand-written kernels.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+SUPPORTED_GROUP_SIZES = (32, 64, 128)
+MLX_BITS = (2, 3, 4, 5, 6, 8)  # what mx.quantize accepts
+SUPPORTED_BITS = (4, 8)  # what this build has kernels for
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check_mode(fn: str, mode: str) -> None:
+    if mode != "affine":
+        raise ValueError(f"[{fn}] Invalid quantization mode '{mode}': this build implements 'affine' only.")
+
+
+def _check_group_bits(fn: str, group_size: int, bits: int) -> None:
+    if group_size not in SUPPORTED_GROUP_SIZES:
+        raise ValueError(
+            f"[{fn}] The requested group size {group_size} is not supported. "
+            "The supported group sizes are 32, 64, and 128."
+        )
+    if bits not in MLX_BITS:
+        raise ValueError(
+            f"[{fn}] The requested number of bits {bits} is not supported. "
+            "The supported bits are 2, 3, 4, 5, 6 and 8."
+        )
+    if bits not in SUPPORTED_BITS:
+        raise ValueError(f"[{fn}] {bits}-bit packing is not implemented in this build (4 and 8 are).")
+
+
+def _require_hip(fn: str, t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"[{fn}] `{name}` lives on {t.device}; the mfq kernels run on a HIP device only "
+            "and there is no CPU fallback."
+        )
+
+
+def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4, mode: str = "affine"):
+    """Group-wise affine quantization of the last axis of ``w``.
+
+    Returns ``(w_q, scales, biases)``: ``w_q`` uint32 ``[..., K*bits/32]`` with
+    element ``i`` of each word at bit offset ``i*bits``; ``scales``/``biases`` of
+    ``w``'s dtype, ``[..., K/group_size]``.  Bit-identical to MLX's CPU result.
+    """
+    _check_mode("quantize", mode)
+    _check_group_bits("quantize", group_size, bits)
+    if w.dtype not in _DTYPE_CODE:
+        raise ValueError(f"[quantize] Only floating point inputs are supported but got {w.dtype}.")
+    if w.ndim < 2:
+        raise ValueError(
+            f"[quantize] The matrix to be quantized must have at least 2 dimension but it has only {w.ndim}."
+        )
+    K = w.shape[-1]
+    if K % group_size != 0:
+        raise ValueError(
+            "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
+            f"group size {group_size}. However the provided matrix has shape {tuple(w.shape)}"
+        )
+    _require_hip("quantize", w, "w")
+    w = w.contiguous()
+    lead = tuple(w.shape[:-1])
+    rows = w.numel() // K
+    wq = torch.empty((*lead, K * bits // 32), dtype=torch.uint32, device=w.device)
+    scales = torch.empty((*lead, K // group_size), dtype=w.dtype, device=w.device)
+    biases = torch.empty_like(scales)
+    with torch.cuda.device(w.device):
+        rc = _lib.load().mfq_quantize_affine(
+            w.data_ptr(), _DTYPE_CODE[w.dtype], rows, K, group_size, bits,
+            wq.data_ptr(), scales.data_ptr(), biases.data_ptr(), _stream_ptr(w.device),
+        )
+    _lib.check("mfq_quantize_affine", rc)
+    return wq, scales, biases
+
+
+def _check_packed(fn: str, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int, bits: int):
+    if w.dtype != torch.uint32:
+        raise ValueError(f"[{fn}] The weight matrix should be uint32 but received {w.dtype}")
+    if scales.shape != biases.shape:
+        raise ValueError(f"[{fn}] Scales and biases should have the same shape. Received scales with shape "
+                         f"{tuple(scales.shape)} and biases with {tuple(biases.shape)}")
+    if scales.dtype != biases.dtype or scales.dtype not in _DTYPE_CODE:
+        raise ValueError(f"[{fn}] Scales and biases must share a floating point dtype, got {scales.dtype} "
+                         f"and {biases.dtype}")
+    if w.ndim < 2 or w.shape[:-1] != scales.shape[:-1]:
+        raise ValueError(f"[{fn}] Weight, scales and biases should have the same batch shape. Received weight "
+                         f"with shape {tuple(w.shape)}, scales with {tuple(scales.shape)}")
+    if w.shape[-1] * 32 // bits != scales.shape[-1] * group_size:
+        raise ValueError(
+            f"[{fn}] The shapes of the weight and scales are incompatible based on bits and group_size. "
+            f"w.shape() == {tuple(w.shape)} and scales.shape() == {tuple(scales.shape)} "
+            f"with group_size={group_size} and bits={bits}"
+        )
+
+
+def dequantize(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64, bits: int = 4,
+               mode: str = "affine", dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``code * scale + bias`` in ``dtype`` (default: the dtype of ``scales``).
+    The value is the float32 fused multiply-add rounded once."""
+    _check_mode("dequantize", mode)
+    _check_group_bits("dequantize", group_size, bits)
+    _check_packed("dequantize", w, scales, biases, group_size, bits)
+    _require_hip("dequantize", w, "w")
+    out_dtype = scales.dtype if dtype is None else dtype
+    if out_dtype not in (scales.dtype, torch.float32):
+        raise ValueError(f"[dequantize] Output dtype must be {scales.dtype} or float32, got {out_dtype}")
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    K = w.shape[-1] * 32 // bits
+    rows = w.numel() // w.shape[-1]
+    out = torch.empty((*w.shape[:-1], K), dtype=out_dtype, device=w.device)
+    with torch.cuda.device(w.device):
+        rc = _lib.load().mfq_dequantize_affine(
+            w.data_ptr(), scales.data_ptr(), biases.data_ptr(), _DTYPE_CODE[scales.dtype], rows, K, group_size, bits,
+            out.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(w.device),
+        )
+    _lib.check("mfq_dequantize_affine", rc)
+    return out
+
+
+def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                     transpose: bool = True, group_size: int = 64, bits: int = 4, mode: str = "affine",
+                     *, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ dequantize(w).T`` with float32 accumulation.
+
+    ``x``: ``[..., K]``; ``w``: packed ``[N, K*bits/32]``.  The result has dtype
+    ``result_type(x, scales)``; when that is float32 (float32 ``x`` against
+    16-bit scales) ``x`` is rounded to the dtype of ``scales`` for the matrix
+    cores and only the accumulation and output are float32.  ``bias`` (not part
+    of ``mx.quantized_matmul``) fuses the add of ``QuantizedLinear`` into the
+    kernel's epilogue with the same two roundings as a separate add.
+    """
+    _check_mode("quantized_matmul", mode)
+    _check_group_bits("quantized_matmul", group_size, bits)
+    if not transpose:
+        raise NotImplementedError("[quantized_matmul] transpose=False (x @ w) is not implemented in this build")
+    _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
+    if w.ndim != 2:
+        raise NotImplementedError("[quantized_matmul] batched weights are not implemented in this build")
+    if x.dtype not in _DTYPE_CODE:
+        raise ValueError(f"[quantized_matmul] Only real floating types are supported but {x.dtype} was provided "
+                         "for the input")
+    if scales.dtype == torch.float32:
+        raise NotImplementedError("[quantized_matmul] float32 scales are not implemented in this build")
+    N = w.shape[0]
+    K = w.shape[1] * 32 // bits
+    if x.ndim < 1 or x.shape[-1] != K:
+        raise ValueError(
+            f"[quantized_matmul] Last dimension of first input with shape {tuple(x.shape)} does not match the "
+            f"expanded quantized matrix ({K}, {N}) computed from shape {tuple(w.shape)} with "
+            f"group_size={group_size}, bits={bits} and transpose=true"
+        )
+    _require_hip("quantized_matmul", x, "x")
+    _require_hip("quantized_matmul", w, "w")
+    out_dtype = torch.result_type(x, scales)
+    compute = scales.dtype
+    lead = tuple(x.shape[:-1])
+    x2 = x.reshape(-1, K)
+    if x2.dtype != compute:
+        x2 = x2.to(compute)
+    x2 = x2.contiguous()
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    if M == 0:
+        return y.reshape(*lead, N)
+    if bias is not None:
+        if bias.shape != (N,):
+            raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
+        bias = bias.to(compute).contiguous()
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    with torch.cuda.device(x.device):
+        rc = _lib.load().mfq_qmm_t(
+            x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+            _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
+            y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device),
+        )
+    _lib.check("mfq_qmm_t", rc)
+    return y.reshape(*lead, N)

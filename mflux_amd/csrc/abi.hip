@@ -1,0 +1,77 @@
+// C ABI of libmfq.so: argument validation and dispatch.  No kernel is
+// launched unless every check has passed, so a caller's mistake is an error
+// code and never a device fault.
+#include "common.h"
+
+namespace {
+
+int check_common(int gs, int bits) {
+  if (gs != 32 && gs != 64 && gs != 128) return MFQ_EGROUP;
+  if (bits != 4 && bits != 8) return MFQ_EBITS;
+  return MFQ_OK;
+}
+
+bool is16(int dtype) { return dtype == MFQ_BF16 || dtype == MFQ_F16; }
+bool known(int dtype) { return dtype == MFQ_F32 || is16(dtype); }
+
+}  // namespace
+
+extern "C" {
+
+int mfq_version(void) { return 100; }
+
+const char* mfq_strerror(int status) {
+  switch (status) {
+    case MFQ_OK: return "ok";
+    case MFQ_EDTYPE: return "unsupported dtype";
+    case MFQ_EGROUP: return "group_size must be 32, 64 or 128";
+    case MFQ_EBITS: return "bits must be 4 or 8";
+    case MFQ_ESHAPE: return "bad shape: sizes must be positive and K a multiple of group_size";
+    case MFQ_ENULL: return "null pointer";
+    case MFQ_EALIGN: return "buffers must be 16-byte aligned";
+    case MFQ_ELAUNCH: return "HIP launch failed";
+    case MFQ_EUNSUPPORTED: return "no kernel for this combination";
+    default: return "unknown status";
+  }
+}
+
+int mfq_quantize_affine(const void* w, int dtype, int64_t rows, int64_t K, int group_size, int bits, uint32_t* wq,
+                        void* scales, void* biases, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!known(dtype)) return MFQ_EDTYPE;
+  if (rows <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (!w || !wq || !scales || !biases) return MFQ_ENULL;
+  if (!mfq::aligned16(w) || !mfq::aligned16(wq)) return MFQ_EALIGN;
+  return mfq::launch_quantize(w, dtype, rows, K, group_size, bits, wq, scales, biases, (hipStream_t)stream);
+}
+
+int mfq_dequantize_affine(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype, int64_t rows,
+                          int64_t K, int group_size, int bits, void* out, int out_dtype, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!known(sb_dtype) || !known(out_dtype)) return MFQ_EDTYPE;
+  if (rows <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (!wq || !scales || !biases || !out) return MFQ_ENULL;
+  if (!mfq::aligned16(wq) || !mfq::aligned16(out)) return MFQ_EALIGN;
+  return mfq::launch_dequantize(wq, scales, biases, sb_dtype, rows, K, group_size, bits, out, out_dtype,
+                                (hipStream_t)stream);
+}
+
+int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+              const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
+              int y_dtype, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
+  if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
+  if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
+  if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
+  if (M <= 16)
+    return mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                           (hipStream_t)stream);
+  if (K % 64) return MFQ_EUNSUPPORTED;
+  return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                         (hipStream_t)stream);
+}
+
+}  // extern "C"

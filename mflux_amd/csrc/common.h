@@ -1,0 +1,129 @@
+// Shared device/host helpers for the mfq kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mfq.h"
+
+namespace mfq {
+
+constexpr int kWave = 64;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Storage element tags.  `bits16` types travel as raw uint16_t in packed
+// registers; conversions are explicit so that rounding points are visible.
+struct BF16 {
+  using storage = uint16_t;
+  using vec8 = bf16x8;
+  static constexpr int code = MFQ_BF16;
+  __device__ static inline float to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+  // round to nearest even; the compiler selects v_cvt_pk_bf16_f32 for pairs
+  __device__ static inline uint16_t from_f32(float f) {
+    __bf16 b = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, b);
+  }
+  __device__ static inline uint32_t pack2(float lo, float hi) {
+    bf16x2 v;
+    v[0] = (__bf16)lo;
+    v[1] = (__bf16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+  }
+};
+
+struct F16 {
+  using storage = uint16_t;
+  using vec8 = f16x8;
+  static constexpr int code = MFQ_F16;
+  __device__ static inline float to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+  __device__ static inline uint16_t from_f32(float f) {
+    _Float16 b = (_Float16)f;
+    return __builtin_bit_cast(uint16_t, b);
+  }
+  __device__ static inline uint32_t pack2(float lo, float hi) {
+    f16x2 v;
+    v[0] = (_Float16)lo;
+    v[1] = (_Float16)hi;
+    return __builtin_bit_cast(uint32_t, v);
+  }
+};
+
+// Matrix-core wrappers.  16x16x32: lane l holds row/col l%16 and the 8
+// consecutive k values starting at 8*(l/16); the result holds rows
+// 4*(l/16)+i (i = 0..3) of column l%16.  32x32x16: lane l holds row/col l%32
+// and k values 8*(l/32)..+7; result register i is row 8*(i/4)+4*(l/32)+i%4 of
+// column l%32.
+__device__ inline f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ inline f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+__device__ inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ inline f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+struct F32 {
+  using storage = float;
+  static constexpr int code = MFQ_F32;
+  __device__ static inline float to_f32(float f) { return f; }
+  __device__ static inline float from_f32(float f) { return f; }
+};
+
+// low / high half of a packed pair of 16-bit elements
+template <typename T>
+__device__ inline float lo_f32(uint32_t p) { return T::to_f32((uint16_t)(p & 0xffffu)); }
+template <typename T>
+__device__ inline float hi_f32(uint32_t p) { return T::to_f32((uint16_t)(p >> 16)); }
+
+// byte j of a word as float (selects v_cvt_f32_ubyte{j})
+__device__ inline float ubyte_f32(uint32_t w, int j) { return (float)((w >> (8 * j)) & 0xffu); }
+
+// Dequantise 8 consecutive codes into 8 packed 16-bit elements:
+// value = fma(code, scale, bias) in float32, rounded once to T.
+template <typename T>
+__device__ inline uint4 dequant8_w4(uint32_t word, float s, float b) {
+  const uint32_t even = word & 0x0f0f0f0fu;         // codes 0,2,4,6 in bytes 0..3
+  const uint32_t odd = (word >> 4) & 0x0f0f0f0fu;   // codes 1,3,5,7
+  uint4 r;
+  r.x = T::pack2(__builtin_fmaf(ubyte_f32(even, 0), s, b), __builtin_fmaf(ubyte_f32(odd, 0), s, b));
+  r.y = T::pack2(__builtin_fmaf(ubyte_f32(even, 1), s, b), __builtin_fmaf(ubyte_f32(odd, 1), s, b));
+  r.z = T::pack2(__builtin_fmaf(ubyte_f32(even, 2), s, b), __builtin_fmaf(ubyte_f32(odd, 2), s, b));
+  r.w = T::pack2(__builtin_fmaf(ubyte_f32(even, 3), s, b), __builtin_fmaf(ubyte_f32(odd, 3), s, b));
+  return r;
+}
+
+template <typename T>
+__device__ inline uint4 dequant8_w8(uint32_t w0, uint32_t w1, float s, float b) {
+  uint4 r;
+  r.x = T::pack2(__builtin_fmaf(ubyte_f32(w0, 0), s, b), __builtin_fmaf(ubyte_f32(w0, 1), s, b));
+  r.y = T::pack2(__builtin_fmaf(ubyte_f32(w0, 2), s, b), __builtin_fmaf(ubyte_f32(w0, 3), s, b));
+  r.z = T::pack2(__builtin_fmaf(ubyte_f32(w1, 0), s, b), __builtin_fmaf(ubyte_f32(w1, 1), s, b));
+  r.w = T::pack2(__builtin_fmaf(ubyte_f32(w1, 2), s, b), __builtin_fmaf(ubyte_f32(w1, 3), s, b));
+  return r;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Entry points of the individual translation units (host side).
+int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, int bits, uint32_t* wq,
+                    void* scales, void* biases, hipStream_t stream);
+int launch_dequantize(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype, int64_t rows,
+                      int64_t K, int gs, int bits, void* out, int out_dtype, hipStream_t stream);
+int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+               const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+               hipStream_t stream);
+int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+               const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+               hipStream_t stream);
+
+}  // namespace mfq

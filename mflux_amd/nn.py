@@ -1,0 +1,149 @@
+"""Module-level API: ``quantize``, ``QuantizedLinear``, ``Linear``.
+
+Mirrors the part of ``mlx.nn`` that mflux uses to quantize a model and to run
+it: ``nn.quantize(model, class_predicate=..., bits=...)`` at
+src/mflux/models/common/weights/loading/weight_applier.py:43,46,103, the
+``hasattr(module, "to_quantized")`` predicates
+(src/mflux/models/flux/weights/flux_weight_definition.py:79-81) and the
+attributes the LoRA wrappers read from a quantized layer
+(src/mflux/models/common/lora/layer/linear_lora_layer.py:14-16:
+``weight.shape == (N, K*bits/32)`` and ``bits``).
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable
+
+import torch
+
+from . import core
+
+
+def _defaults(group_size: int | None, bits: int | None) -> tuple[int, int]:
+    return (64 if group_size is None else group_size, 4 if bits is None else bits)
+
+
+class QuantizedLinear(torch.nn.Module):
+    """``y = quantized_matmul(x, weight, scales, biases) (+ bias)``.
+
+    Tensors are named as MLX names them (``weight`` packed uint32
+    ``[N, K*bits/32]``, ``scales``/``biases`` ``[N, K/group_size]``, optional
+    ``bias`` ``[N]``) and are frozen (buffers, no gradient), so
+    ``state_dict()`` is exactly what mflux saves for the layer.
+    """
+
+    def __init__(self, input_dims: int, output_dims: int, bias: bool = True, group_size: int | None = None,
+                 bits: int | None = None, mode: str = "affine", *, device=None, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        self.group_size, self.bits = _defaults(group_size, bits)
+        self.mode = mode
+        core._check_mode("QuantizedLinear", mode)
+        core._check_group_bits("QuantizedLinear", self.group_size, self.bits)
+        if input_dims % self.group_size:
+            raise ValueError(
+                "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
+                f"group size {self.group_size}. However the provided matrix has shape {(output_dims, input_dims)}"
+            )
+        device = torch.device("cpu" if device is None else device)
+        if device.type == "cuda":
+            bound = math.sqrt(1.0 / input_dims)
+            w = torch.empty((output_dims, input_dims), device=device, dtype=torch.float32).uniform_(-bound, bound)
+            wq, scales, biases = core.quantize(w.to(dtype), self.group_size, self.bits)
+        else:  # placeholders of the right shape, to be filled by load_state_dict / update
+            wq = torch.zeros((output_dims, input_dims * self.bits // 32), dtype=torch.uint32, device=device)
+            scales = torch.zeros((output_dims, input_dims // self.group_size), dtype=dtype, device=device)
+            biases = torch.zeros_like(scales)
+        self.register_buffer("weight", wq)
+        self.register_buffer("scales", scales)
+        self.register_buffer("biases", biases)
+        if bias:
+            self.register_buffer("bias", torch.zeros((output_dims,), dtype=dtype, device=device))
+        else:
+            self.bias = None
+
+    @property
+    def input_dims(self) -> int:
+        return self.weight.shape[1] * 32 // self.bits
+
+    @property
+    def output_dims(self) -> int:
+        return self.weight.shape[0]
+
+    def extra_repr(self) -> str:
+        return (f"input_dims={self.input_dims}, output_dims={self.output_dims}, bias={self.bias is not None}, "
+                f"group_size={self.group_size}, bits={self.bits}, mode={self.mode}")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return core.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                     group_size=self.group_size, bits=self.bits, mode=self.mode, bias=self.bias)
+
+    @classmethod
+    def from_linear(cls, linear_layer: torch.nn.Module, group_size: int | None = None, bits: int | None = None,
+                    mode: str = "affine") -> "QuantizedLinear":
+        weight = linear_layer.weight.detach()
+        output_dims, input_dims = weight.shape
+        group_size, bits = _defaults(group_size, bits)
+        ql = cls.__new__(cls)
+        torch.nn.Module.__init__(ql)
+        ql.group_size, ql.bits, ql.mode = group_size, bits, mode
+        wq, scales, biases = core.quantize(weight, group_size, bits, mode)
+        ql.register_buffer("weight", wq)
+        ql.register_buffer("scales", scales)
+        ql.register_buffer("biases", biases)
+        lin_bias = getattr(linear_layer, "bias", None)
+        if lin_bias is not None:
+            ql.register_buffer("bias", lin_bias.detach())
+        else:
+            ql.bias = None
+        return ql
+
+
+class Linear(torch.nn.Linear):
+    """``torch.nn.Linear`` with MLX's ``to_quantized`` hook, so that the
+    reference's ``hasattr(module, "to_quantized")`` predicates select it."""
+
+    def to_quantized(self, group_size: int | None = None, bits: int | None = None, mode: str = "affine"):
+        return QuantizedLinear.from_linear(self, group_size, bits, mode)
+
+
+def leaf_modules(model: torch.nn.Module):
+    """(dotted path, parent, attribute name, module) of every module without
+    children, in registration order -- MLX's ``Module.leaf_modules()`` with the
+    same path spelling (``blocks.0.attn.to_q``)."""
+    out = []
+    for path, module in model.named_modules():
+        if path == "" or any(True for _ in module.children()):
+            continue
+        parent_path, _, name = path.rpartition(".")
+        parent = model.get_submodule(parent_path) if parent_path else model
+        out.append((path, parent, name, module))
+    return out
+
+
+def quantize(model: torch.nn.Module, group_size: int | None = None, bits: int | None = None, *,
+             mode: str = "affine", class_predicate: Callable | None = None) -> torch.nn.Module:
+    """Replaces, in place, every leaf module the predicate selects by its
+    quantized counterpart (``module.to_quantized(...)``).
+
+    ``class_predicate(path, module)`` returns a bool, or a dict of keyword
+    arguments for ``to_quantized``.  The default selects every module that has a
+    ``to_quantized`` method.  A truthy answer for a module without one raises
+    ``ValueError``.  Returns the model.
+    """
+    group_size, bits = _defaults(group_size, bits)
+    class_predicate = class_predicate or (lambda _, m: hasattr(m, "to_quantized"))
+    for path, parent, name, module in leaf_modules(model):
+        answer = class_predicate(path, module)
+        if not answer:
+            continue
+        if not hasattr(module, "to_quantized"):
+            raise ValueError(f"Unable to quantize model of type {type(module)}")
+        if isinstance(answer, bool):
+            kwargs = {"group_size": group_size, "bits": bits, "mode": mode}
+        elif isinstance(answer, dict):
+            kwargs = answer
+        else:
+            raise ValueError("``class_predicate`` must return a bool or a dict of parameters to pass to "
+                             "``to_quantized``")
+        parent._modules[name] = module.to_quantized(**kwargs)
+    return model

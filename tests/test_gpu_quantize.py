@@ -1,0 +1,150 @@
+"""GPU parity: libmfq's quantize / dequantize against the CPU oracle,
+bit for bit, through the C ABI (ctypes)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def _adversarial_groups(o, n_groups: int, gs: int, seed: int) -> np.ndarray:
+    """float32 rows of groups built to hit the corners of the algorithm:
+    ties at x.5 code boundaries, all-equal groups, zeros of both signs, tiny
+    values under the eps clamp, denormals, a huge dynamic range, max-only and
+    min-only edges."""
+    rng = np.random.default_rng(seed)
+    g = np.empty((n_groups, gs), dtype=np.float32)
+    for i in range(n_groups):
+        kind = i % 12
+        if kind == 0:   # exact grid: codes land on integers and on .5 ties
+            step = np.float32(2.0 ** rng.integers(-12, 4))
+            g[i] = rng.integers(-15, 16, gs).astype(np.float32) * step * np.float32(0.5)
+        elif kind == 1:  # all equal
+            g[i] = np.float32(rng.standard_normal() * 0.02)
+        elif kind == 2:  # zeros of both signs
+            g[i] = np.where(rng.random(gs) < 0.5, np.float32(0.0), np.float32(-0.0))
+        elif kind == 3:  # below the eps clamp
+            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e-8)
+        elif kind == 4:  # float32 denormals (flush to zero in bf16 inputs, kept for f32)
+            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e-40)
+        elif kind == 5:  # huge dynamic range
+            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(10.0) ** rng.integers(-6, 6, gs).astype(np.float32)
+        elif kind == 6:  # all positive: the maximum is the edge
+            g[i] = np.abs(rng.standard_normal(gs)).astype(np.float32)
+        elif kind == 7:  # all negative: the minimum is the edge
+            g[i] = -np.abs(rng.standard_normal(gs)).astype(np.float32)
+        elif kind == 8:  # |min| == |max|
+            v = rng.standard_normal(gs).astype(np.float32)
+            v[0], v[1] = np.float32(-3.0), np.float32(3.0)
+            g[i] = np.clip(v, -3, 3)
+        elif kind == 9:  # one outlier
+            v = rng.standard_normal(gs).astype(np.float32) * np.float32(0.01)
+            v[rng.integers(gs)] = np.float32(50.0)
+            g[i] = v
+        elif kind == 10:  # large magnitudes
+            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e30)
+        else:
+            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(0.02)
+    return g
+
+
+def _storage(o, f32: np.ndarray, dtype: int) -> np.ndarray:
+    if dtype == o.BF16:
+        return o.f32_to_bf16_bits(f32)
+    if dtype == o.F16:
+        with np.errstate(over="ignore"):
+            h = np.clip(f32, -60000, 60000).astype(np.float16)
+        return h.view(np.uint16)
+    return f32
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16", "f32"])
+def test_quantize_bit_exact_random_and_adversarial(oracle, bits, gs, dtype_name):
+    import mflux_amd
+    from gpu_util import raw, to_dev
+
+    o = oracle
+    dtype = {"bf16": o.BF16, "f16": o.F16, "f32": o.F32}[dtype_name]
+    rows, K = 96, 1024
+    rnd = seeded(9, bits * 1000 + gs, (rows, K), 0.02)
+    adv = _adversarial_groups(o, rows * K // gs, gs, seed=bits + gs).reshape(rows, K)
+    for name, f32 in (("random", rnd), ("adversarial", adv)):
+        w = _storage(o, f32, dtype)
+        exp = o.c_quantize(w, dtype, gs, bits)
+        got = mflux_amd.quantize(to_dev(w, dtype), group_size=gs, bits=bits)
+        torch.cuda.synchronize()
+        for what, e, g in zip(("wq", "scales", "biases"), exp, got):
+            assert tuple(g.shape) == e.shape, (name, what)
+            ge = raw(g)
+            bad = np.flatnonzero(ge.reshape(-1) != e.reshape(-1))
+            assert bad.size == 0, f"{name}/{what}: {bad.size} mismatches, first at {bad[:4]}"
+
+
+@pytest.mark.parametrize("bits,N,K", [(4, 3072, 3072), (8, 2048, 3072), (4, 1024, 15360)])
+def test_quantize_bit_exact_model_shapes(oracle, bits, N, K):
+    import mflux_amd
+    from gpu_util import raw, to_dev
+
+    o = oracle
+    w = o.f32_to_bf16_bits(seeded(3, bits, (N, K), 0.02))
+    exp = o.c_quantize(w, o.BF16, 64, bits)
+    got = mflux_amd.quantize(to_dev(w, o.BF16), group_size=64, bits=bits)
+    for e, g in zip(exp, got):
+        assert np.array_equal(raw(g), e)
+
+
+def test_quantize_leading_dims_and_tail(oracle):
+    """3-D input and a chunk count that does not fill the last wavefront."""
+    import mflux_amd
+    from gpu_util import raw, to_dev
+
+    o = oracle
+    w = o.f32_to_bf16_bits(seeded(9, 77, (3, 5, 96), 1.0))
+    exp = o.c_quantize(w, o.BF16, 32, 4)
+    got = mflux_amd.quantize(to_dev(w, o.BF16), group_size=32, bits=4)
+    for e, g in zip(exp, got):
+        assert tuple(g.shape) == e.shape
+        assert np.array_equal(raw(g), e)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_dequantize_single_rounding(oracle, bits, gs):
+    """dequantize == float32 fma(code, scale, bias) rounded once to bf16, and
+    exact in float32 output for bf16 scales where the sum fits 24 bits."""
+    import mflux_amd
+    from gpu_util import raw, to_dev, u32_to_dev
+
+    o = oracle
+    w = o.f32_to_bf16_bits(seeded(9, 5, (64, 1024), 0.02))
+    wq, s, b = o.c_quantize(w, o.BF16, gs, bits)
+    exact = o.dequantize_exact(wq, s, b, o.BF16, gs, bits)
+    fma32 = exact.astype(np.float32)  # correctly rounded float32 of the exact value == fmaf
+    exp_bf16 = o.f32_to_bf16_bits(fma32)
+    d = mflux_amd.dequantize(u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16), group_size=gs, bits=bits)
+    assert d.dtype == torch.bfloat16
+    assert np.array_equal(raw(d), exp_bf16)
+    d32 = mflux_amd.dequantize(u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16), group_size=gs, bits=bits,
+                               dtype=torch.float32)
+    assert np.array_equal(raw(d32), fma32)
+
+
+def test_quantize_dequantize_error_bound_full_size():
+    """At the full single-block shape the dequantised weight is within
+    |scale|/2 of the input (plus the bf16 rounding of the stored scale, at most
+    n_bins * 2^-9 * |scale|), and codes stay inside [0, n_bins]."""
+    import mflux_amd
+
+    torch.manual_seed(3001)
+    w = (torch.randn(21504, 3072, device="cuda") * 0.02).to(torch.bfloat16)
+    wq, s, b = mflux_amd.quantize(w, 64, 4)
+    d = mflux_amd.dequantize(wq, s, b, 64, 4, dtype=torch.float32)
+    err = (d - w.float()).abs().reshape(21504, 48, 64)
+    bound = s.float().abs().reshape(21504, 48, 1) * (0.5 + 15 * 2.0 ** -9) + 1e-12
+    assert bool((err <= bound).all())
+    # every group reproduces its edge element exactly (bias is the edge, code 0)
+    assert bool((err.amin(dim=2) == 0).all())
