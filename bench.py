@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Step = one pass of the FLUX.1 single-stream block's quantized linears at
+1024x1024 (BASELINE config 3): x[4608,3072] @ W4[21504,3072]^T followed by
+x2[4608,15360] @ W4[3072,15360]^T, group size 64, bf16 activations, synthetic
+N(0,1) activations and N(0,0.02) weights quantized on the device by this
+library.  Prints ONE JSON line; `value` is TFLOP/s over the two GEMMs with all
+operands resident in HBM.
+
+The same line carries
+  roofline     - the W4A16 GEMM kernel against the dense bf16 MFMA peak, from
+                 HIP-event timing of the launches in the timed region;
+  secondary    - the W8 dequant-GEMV (BASELINE config 2, M=1 and M=4) against
+                 the HBM peak, weights rotated through > 256 MB so the memory-
+                 side cache cannot serve them, and the quantize/pack pass over
+                 both block weights;
+  cpu_baseline - the CPU oracle's scalar qmm (a port of MLX's CPU loop; MLX
+                 itself cannot be installed here) on a bounded row sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+M_TOKENS = 4608
+LINEARS = (("linear1", 3072, 21504), ("linear2", 15360, 3072))  # (name, K, N)
+GS, BITS = 64, 4
+
+
+def qmm_bytes(M, K, N, bits, bias=False):
+    return N * K * bits // 8 + 4 * N * K // 64 + 2 * M * K + 2 * M * N + (2 * N if bias else 0)
+
+
+def quantize_bytes(N, K, bits):
+    return 2 * N * K + N * K * bits // 8 + 4 * N * K // 64
+
+
+def event_ms(fn, iters, torch):
+    """Average milliseconds per call of fn over `iters` back-to-back calls,
+    measured with HIP events on the current stream (the stream fn launches on)."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def graph_ms(fn, calls, replays, torch):
+    """Average milliseconds per call of fn with `calls` calls captured into one
+    HIP graph and replayed `replays` times: back-to-back kernels without the
+    host's per-call launch cost, which would otherwise dominate a ~10 us kernel.
+    Events are recorded on the stream the graph replays on."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / (calls * replays)
+
+
+def cpu_baseline(torch, x, wq, s, b, sample_rows):
+    """Times the oracle's scalar qmm_t (float32 accumulation) on the first
+    `sample_rows` rows of the linear1 problem, on all host threads and on one."""
+    import numpy as np
+    from oracle import mlx_affine as o
+
+    def raw16(t):
+        return t.contiguous().cpu().view(torch.int16).numpy().view(np.uint16)
+
+    xs = raw16(x[:sample_rows])
+    wq_h = wq.cpu().view(torch.int32).numpy().view(np.uint32)
+    s_h, b_h = raw16(s), raw16(b)
+    N, K = wq_h.shape[0], xs.shape[1]
+    threads = min(o.num_threads(), len(os.sched_getaffinity(0)))
+    flops = 2.0 * sample_rows * N * K
+    t0 = time.perf_counter()
+    o.c_qmm_t(xs, o.BF16, wq_h, s_h, b_h, o.BF16, None, GS, BITS, threads=threads)
+    t_all = time.perf_counter() - t0
+    one_rows = max(1, sample_rows // 8)
+    t0 = time.perf_counter()
+    o.c_qmm_t(xs[:one_rows], o.BF16, wq_h, s_h, b_h, o.BF16, None, GS, BITS, threads=1)
+    t_one = time.perf_counter() - t0
+    return {
+        "value": round(flops / t_all / 1e12, 6),
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {sample_rows} of {M_TOKENS} rows of linear1 (K=3072, N=21504, W4 gs64), "
+                  f"{t_all:.1f} s on {threads} threads; scalar float32-accumulating port of MLX's CPU _qmm_t "
+                  "(MLX is not installable offline)",
+        "single_thread_value": round(2.0 * one_rows * N * K / t_one / 1e12, 6),
+        "single_thread_sample": f"first {one_rows} rows, {t_one:.1f} s on 1 thread",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-rows", type=int, default=512)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (--gpus 1); nothing is sharded across devices")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible")
+    import mflux_amd
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(3000)
+
+    # ---- operands of the step, resident in HBM --------------------------------
+    ops = []
+    quant_ms = {}
+    for name, K, N in LINEARS:
+        x = torch.randn(M_TOKENS, K, device=dev, generator=gen).to(torch.bfloat16)
+        w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        wq, s, b = mflux_amd.quantize(w, GS, BITS)
+        copies = [w] + [w.clone() for _ in range(3)]  # > 256 MB in rotation: cold reads
+        turn = {"i": 0}
+
+        def quantize_call():
+            turn["i"] += 1
+            mflux_amd.quantize(copies[turn["i"] % len(copies)], GS, BITS)
+
+        quant_ms[name] = graph_ms(quantize_call, 8, 5, torch)
+        del copies, w
+        ops.append((name, x, wq, s, b))
+
+    def step():
+        for _, x, wq, s, b in ops:
+            mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=BITS)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    kernel_ms_per_step = start.elapsed_time(stop) / args.steps
+
+    flops = sum(2.0 * M_TOKENS * K * N for _, K, N in LINEARS)
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    launches = len(LINEARS)
+    achieved = flops / (kernel_ms_per_step * 1e-3) / 1e12  # = mean flops per launch / mean launch duration
+    roofline = {
+        "kernel": "qmm_kernel<BF16,64,4>",
+        "bound": "mfma",
+        "achieved": round(achieved, 2),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+        "traffic": None,
+        "avg_launch_us": round(kernel_ms_per_step * 1e3 / launches, 2),
+        "flops_per_launch": flops / launches,
+    }
+
+    # per-shape GEMM timings
+    per_shape = {}
+    for name, x, wq, s, b in ops:
+        ms = event_ms(lambda: mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=BITS), 20, torch)
+        K, N = x.shape[1], wq.shape[0]
+        per_shape[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
+
+    # ---- secondary: W8 GEMV (config 2), cold weights ---------------------------
+    gemv = {}
+    Kg, Ng = 3072, 18432
+    n_buf = 8
+    bufs = []
+    for i in range(n_buf):
+        w = (torch.randn(Ng, Kg, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        bufs.append(mflux_amd.quantize(w, GS, 8))
+        del w
+    bias = (torch.randn(Ng, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    for Mg in (1, 4):
+        temb = torch.randn(Mg, Kg, device=dev, generator=gen)
+        xg = torch.nn.functional.silu(temb).to(torch.bfloat16)
+        state = {"i": 0}
+
+        def gemv_call():
+            wq8, s8, b8 = bufs[state["i"] % n_buf]
+            state["i"] += 1
+            mflux_amd.quantized_matmul(xg, wq8, s8, b8, group_size=GS, bits=8, bias=bias)
+
+        state["i"] = 0
+        ms = graph_ms(gemv_call, 4 * n_buf, 10, torch)
+        nbytes = qmm_bytes(Mg, Kg, Ng, 8, bias=True)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        gemv[f"M{Mg}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                          "bytes": nbytes, "weights": f"rotating over {n_buf} buffers ({n_buf * Ng * Kg >> 20} MiB)"}
+    del bufs
+
+    quant = {}
+    for (name, K, N) in LINEARS:
+        ms = quant_ms[name]
+        nbytes = quantize_bytes(N, K, BITS)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        quant[name] = {"us": round(ms * 1e3, 1), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+
+    out = {
+        "metric": "W4A16 qmatmul TFLOP/s @ FLUX single-block M=4608",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "flux1_single_block_1024px_m4608_w4_gs64: linear1 3072->21504 + linear2 15360->3072",
+                   "M": M_TOKENS, "bits": BITS, "group_size": GS},
+        "roofline": roofline,
+        "per_shape": per_shape,
+        "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "gemv_w8": gemv,
+                      "quantize_w4": quant},
+    }
+    if not args.no_cpu_baseline:
+        name, x, wq, s, b = ops[0]
+        out["cpu_baseline"] = cpu_baseline(torch, x, wq, s, b, args.cpu_sample_rows)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -134,9 +134,11 @@ def test_dequantize_single_rounding(oracle, bits, gs):
 
 
 def test_quantize_dequantize_error_bound_full_size():
-    """At the full single-block shape the dequantised weight is within
-    |scale|/2 of the input (plus the bf16 rounding of the stored scale, at most
-    n_bins * 2^-9 * |scale|), and codes stay inside [0, n_bins]."""
+    """At the full single-block shape: every group reproduces its edge element
+    exactly (bias is the edge, code 0); the error of every other element is at
+    most one step (re-fitting the scale to the edge can shrink it by up to
+    1/16, which clips the far end by up to one code) and typically half a
+    step."""
     import mflux_amd
 
     torch.manual_seed(3001)
@@ -144,7 +146,7 @@ def test_quantize_dequantize_error_bound_full_size():
     wq, s, b = mflux_amd.quantize(w, 64, 4)
     d = mflux_amd.dequantize(wq, s, b, 64, 4, dtype=torch.float32)
     err = (d - w.float()).abs().reshape(21504, 48, 64)
-    bound = s.float().abs().reshape(21504, 48, 1) * (0.5 + 15 * 2.0 ** -9) + 1e-12
-    assert bool((err <= bound).all())
-    # every group reproduces its edge element exactly (bias is the edge, code 0)
+    step = s.float().abs().reshape(21504, 48, 1)
+    assert bool((err <= step * (1.0 + 15 * 2.0 ** -9) + 1e-12).all())
+    assert float((err <= step * (0.5 + 15 * 2.0 ** -9)).float().mean()) > 0.99
     assert bool((err.amin(dim=2) == 0).all())
