@@ -4,19 +4,22 @@
 // (e.g. src/mflux/models/flux/model/flux_transformer/
 // single_transformer_block.py:53,57 at M = 4608).
 //
-// One workgroup of four wavefronts computes a 256 x 256 tile of y, each
-// wavefront a 128 x 128 quadrant held as 4 x 4 accumulators of the 32x32x16
-// matrix-core instruction.  Per 64-wide k step:
-//   - x rows go HBM -> registers -> LDS as they are (128-bit moves);
-//   - packed weights go HBM -> registers with 128-bit loads (thread t owns
-//     weight row t of the tile), are dequantised with one float32 fma per code
-//     (single rounding to the 16-bit type) and written to LDS as a second
-//     16-bit tile, so the dequantisation cost is paid once per workgroup and
-//     reused by 256 rows of x;
-//   - global loads for step i+1 are issued before the matrix work of step i
-//     and two LDS buffers alternate, so there is one barrier per step.
-// LDS rows are 128 bytes; the 16-byte column index is XORed with row%8 so both
-// the row-wise writes and the 32-row fragment reads are bank-conflict free.
+// One workgroup of four wavefronts computes a 256 x 256 tile of y; wavefront w
+// owns all 256 rows of output columns [64w, 64w+64) as 8 x 2 accumulators of
+// the 32x32x16 matrix-core instruction.
+//   - x goes HBM -> registers -> LDS (128-bit moves, one 64-wide k step ahead,
+//     two LDS buffers, one barrier per step).  LDS rows are 128 bytes and the
+//     16-byte column index is XORed with row%8, so the row-wise writes and the
+//     32-row fragment reads are both bank-conflict free.
+//   - packed weights never touch LDS: a lane of the matrix core's B operand
+//     holds 8 consecutive k of one output column, which is exactly one uint32
+//     of 4-bit codes (two of 8-bit codes).  Each lane streams 128-bit pieces of
+//     its own weight row straight from HBM/L2 into registers one step ahead and
+//     dequantises a word with one float32 fma per code (single rounding to the
+//     16-bit type) right before the matrix instruction that consumes it.  No
+//     column is dequantised by more than one wavefront.
+//   - the k order inside a step is permuted (lane half h covers k 32h..32h+31)
+//     identically for both operands, which the dot product does not notice.
 #include "common.h"
 
 namespace mfq {
@@ -26,65 +29,42 @@ constexpr int BM = 256;
 constexpr int BN = 256;
 constexpr int BK = 64;
 constexpr int kThreads = 256;
-constexpr int kTileBytes = BM * BK * 2;           // one 16-bit tile: 32 KiB
-constexpr int kLdsBytes = 4 * kTileBytes;         // x and w tiles, double buffered
+constexpr int kTileBytes = BM * BK * 2;   // one 16-bit x tile: 32 KiB
+constexpr int kLdsBytes = 2 * kTileBytes; // double buffered
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ inline int swz(int row, int chunk) { return row * (BK * 2) + ((chunk ^ (row & 7)) << 4); }
 
-template <typename T>
-__device__ inline typename T::vec8 lds_frag(const char* tile, int row, int chunk) {
-  return *reinterpret_cast<const typename T::vec8*>(tile + swz(row, chunk));
-}
-
+// Per-lane stream of packed weights for the wavefront's two 32-column tiles.
 template <typename T, int GS, int BITS>
-struct Loader {
-  static constexpr int kWLoads = BK * BITS / 128;  // 128-bit loads per weight row per step (2 or 4)
-  static constexpr int kGroupsPerStep = (BK + GS - 1) / GS;
+struct WeightRegs {
+  static constexpr int kLoads = BITS / 4;  // 128-bit loads per column tile and step (32 codes per lane)
+  u32x4 w[2][kLoads];
+  float s[2], b[2];
 
-  u32x4 xa[8];
-  u32x4 wv[kWLoads];
-  float s[kGroupsPerStep], b[kGroupsPerStep];
-
-  __device__ inline void issue(const uint16_t* x, const uint32_t* wq, const uint16_t* scales, const uint16_t* biases,
-                               int m0, int n0, int M, int N, int K, int k0) {
-    const int t = threadIdx.x;
+  __device__ inline void issue(const uint32_t* const (&wrow)[2], const uint16_t* const (&srow)[2],
+                               const uint16_t* const (&brow)[2], int k0, int h) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = min(m0 + (t >> 3) + 32 * i, M - 1);
-      xa[i] = *reinterpret_cast<const u32x4*>(x + (int64_t)row * K + k0 + 8 * (t & 7));
-    }
-    const int n = min(n0 + t, N - 1);
-    const u32x4* wrow = reinterpret_cast<const u32x4*>(wq + (int64_t)n * (K * BITS / 32) + k0 * BITS / 32);
+    for (int j = 0; j < 2; ++j) {
+      const u32x4* p = reinterpret_cast<const u32x4*>(wrow[j] + (k0 + 32 * h) * BITS / 32);
 #pragma unroll
-    for (int i = 0; i < kWLoads; ++i) wv[i] = wrow[i];
-    const int64_t g0 = (int64_t)n * (K / GS) + k0 / GS;
-#pragma unroll
-    for (int g = 0; g < kGroupsPerStep; ++g) {
-      s[g] = T::to_f32(scales[g0 + g]);
-      b[g] = T::to_f32(biases[g0 + g]);
+      for (int l = 0; l < kLoads; ++l) w[j][l] = p[l];
+      const int g = (k0 + 32 * h) / GS;
+      s[j] = T::to_f32(srow[j][g]);
+      b[j] = T::to_f32(brow[j][g]);
     }
   }
 
-  __device__ inline void commit(char* xs, char* ws) const {
-    const int t = threadIdx.x;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = (t >> 3) + 32 * i;
-      *reinterpret_cast<u32x4*>(xs + swz(row, t & 7)) = xa[i];
+  // codes 8*sub .. 8*sub+7 of this lane's 32, as 8 dequantised 16-bit values
+  __device__ inline typename T::vec8 frag(int j, int sub) const {
+    uint4 d;
+    if constexpr (BITS == 4) {
+      d = dequant8_w4<T>(w[j][0][sub], s[j], b[j]);
+    } else {
+      d = dequant8_w8<T>(w[j][sub >> 1][(sub & 1) * 2], w[j][sub >> 1][(sub & 1) * 2 + 1], s[j], b[j]);
     }
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {  // chunk c = codes 8c .. 8c+7 of this thread's weight row
-      const int g = (c * 8) / GS;  // 0 unless GS == 32
-      uint4 d;
-      if constexpr (BITS == 4) {
-        d = dequant8_w4<T>(wv[c >> 2][c & 3], s[g], b[g]);
-      } else {
-        d = dequant8_w8<T>(wv[c >> 1][(c & 1) * 2], wv[c >> 1][(c & 1) * 2 + 1], s[g], b[g]);
-      }
-      *reinterpret_cast<uint4*>(ws + swz(t, c)) = d;
-    }
+    return __builtin_bit_cast(typename T::vec8, d);
   }
 };
 
@@ -94,6 +74,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
     int N, int K, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
+  using vec8 = typename T::vec8;
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
   // run of tiles so that neighbours in the run (same weight columns, adjacent
@@ -109,62 +90,108 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   const int m0 = tm * BM;
   const int n0 = tn * BN;
 
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  const int wm = (wave >> 1) * 128;
-  const int wn = (wave & 1) * 128;
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+  const int wn = wave * 64;
   const int r = lane & 31;
   const int h = lane >> 5;
 
-  f32x16 acc[4][4];
+  f32x16 acc[8][2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  Loader<T, GS, BITS> ld;
+  // this lane's two weight rows (columns of y); rows past N are clamped for loads
+  const uint32_t* wrow[2];
+  const uint16_t* srow[2];
+  const uint16_t* brow[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = min(n0 + wn + 32 * j + r, N - 1);
+    wrow[j] = wq + (int64_t)n * (K * BITS / 32);
+    srow[j] = scales + (int64_t)n * (K / GS);
+    brow[j] = biases + (int64_t)n * (K / GS);
+  }
+  // this thread's share of the x tile: 8 rows, one 16-byte column
+  int xoff[8];  // element offsets; M*K < 2^31 is checked by the launcher
+#pragma unroll
+  for (int i = 0; i < 8; ++i) xoff[i] = min(m0 + (t >> 3) + 32 * i, M - 1) * K + 8 * (t & 7);
+
+  u32x4 xa[8];
+  auto issue_x = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(x + xoff[i] + k0);
+  };
+  auto commit_x = [&](char* tile_x) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(tile_x + swz((t >> 3) + 32 * i, t & 7)) = xa[i];
+  };
+
   const int steps = K / BK;
-  ld.issue(x, wq, scales, biases, m0, n0, M, N, K, 0);
-  ld.commit(lds, lds + 2 * kTileBytes);
-  __syncthreads();
+  WeightRegs<T, GS, BITS> wa, wb;
 
-  for (int step = 0; step < steps; ++step) {
-    const int cur = step & 1;
-    const char* xs = lds + cur * kTileBytes;
-    const char* ws = lds + (2 + cur) * kTileBytes;
-    const bool more = step + 1 < steps;
-    if (more) ld.issue(x, wq, scales, biases, m0, n0, M, N, K, (step + 1) * BK);
-
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      typename T::vec8 af[4], bf[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) af[i] = lds_frag<T>(xs, wm + 32 * i + r, 2 * kk + h);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = lds_frag<T>(ws, wn + 32 * j + r, 2 * kk + h);
+  // One k step: prefetch step+1 (x into registers, weights into `next`), run
+  // the matrix work of `step` from LDS buffer step&1 and `now`, then publish
+  // the prefetched x tile.
+  auto do_step = [&](int step, const WeightRegs<T, GS, BITS>& now, WeightRegs<T, GS, BITS>& next) {
+    const char* xs = lds + (step & 1) * kTileBytes;
+    // branch-free prefetch: the last step re-reads its own operands, which nobody consumes
+    const int k_next = min(step + 1, steps - 1) * BK;
+    issue_x(k_next);
+    next.issue(wrow, srow, brow, k_next, h);
+    // Fragment pipeline over 8 slots (4 k sub-steps x 2 halves of the rows):
+    // the LDS reads of slot q+1 are issued before the matrix work of slot q.
+    vec8 af[2][4];
+    auto read_slot = [&](int q, vec8 (&dst)[4]) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
+        dst[i] = *reinterpret_cast<const vec8*>(xs + swz(32 * (4 * (q & 1) + i) + r, 4 * h + (q >> 1)));
+    };
+    read_slot(0, af[0]);
+    vec8 b0, b1;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(af[i], bf[j], acc[i][j]);
+    for (int q = 0; q < 8; ++q) {
+      if (q < 7) read_slot(q + 1, af[(q + 1) & 1]);
+      if ((q & 1) == 0) {
+        b0 = now.frag(0, q >> 1);
+        b1 = now.frag(1, q >> 1);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[4 * (q & 1) + i][0] = mfma32(af[q & 1][i], b0, acc[4 * (q & 1) + i][0]);
+        acc[4 * (q & 1) + i][1] = mfma32(af[q & 1][i], b1, acc[4 * (q & 1) + i][1]);
+      }
     }
-
-    if (more) ld.commit(lds + (cur ^ 1) * kTileBytes, lds + (2 + (cur ^ 1)) * kTileBytes);
+    commit_x(lds + ((step + 1) & 1) * kTileBytes);
     __syncthreads();
+  };
+
+  issue_x(0);
+  wa.issue(wrow, srow, brow, 0, h);
+  commit_x(lds);
+  __syncthreads();
+  int step = 0;
+  for (; step + 1 < steps; step += 2) {  // straight-line body: two steps with the weight registers swapped
+    do_step(step, wa, wb);
+    do_step(step + 1, wb, wa);
   }
+  if (step < steps) do_step(step, wa, wb);
 
   // Epilogue: register e of an accumulator is row 8*(e/4) + 4*h + e%4, column r.
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < 2; ++j) {
     const int col = n0 + wn + 32 * j + r;
     if (col >= N) continue;
     const float bv = bias ? T::to_f32(bias[col]) : 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
+        const int row = m0 + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
         if (row >= M) continue;
         const int64_t o = (int64_t)row * N + col;
         const float v = acc[i][j][e];
@@ -191,6 +218,7 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
       return MFQ_ELAUNCH;
     configured = true;
   }
+  if (M * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;  // 32-bit element offsets into x
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, stream,
