@@ -20,6 +20,8 @@
 //     column is dequantised by more than one wavefront.
 //   - the k order inside a step is permuted (lane half h covers k 32h..32h+31)
 //     identically for both operands, which the dot product does not notice.
+#include <type_traits>
+
 #include "common.h"
 
 namespace mfq {
@@ -43,28 +45,32 @@ struct WeightRegs {
   u32x4 w[2][kLoads];
   float s[2], b[2];
 
-  __device__ inline void issue(const uint32_t* const (&wrow)[2], const uint16_t* const (&srow)[2],
-                               const uint16_t* const (&brow)[2], int k0, int h) {
+  // woff/soff: this lane's byte offsets of its two weight rows / scale rows;
+  // k0 is uniform, so every address is a uniform base plus a 32-bit lane offset.
+  __device__ inline void issue(const uint32_t* wq, const uint16_t* scales, const uint16_t* biases,
+                               const uint32_t (&woff)[2], const uint32_t (&soff)[2], int k0) {
+    const char* wbase = reinterpret_cast<const char*>(wq) + (size_t)k0 * BITS / 8;
+    const char* sbase = reinterpret_cast<const char*>(scales) + (size_t)(k0 / GS) * 2;
+    const char* bbase = reinterpret_cast<const char*>(biases) + (size_t)(k0 / GS) * 2;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const u32x4* p = reinterpret_cast<const u32x4*>(wrow[j] + (k0 + 32 * h) * BITS / 32);
 #pragma unroll
-      for (int l = 0; l < kLoads; ++l) w[j][l] = p[l];
-      const int g = (k0 + 32 * h) / GS;
-      s[j] = T::to_f32(srow[j][g]);
-      b[j] = T::to_f32(brow[j][g]);
+      for (int l = 0; l < kLoads; ++l) w[j][l] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + 16 * l);
+      s[j] = T::to_f32(*reinterpret_cast<const uint16_t*>(sbase + soff[j]));
+      b[j] = T::to_f32(*reinterpret_cast<const uint16_t*>(bbase + soff[j]));
     }
   }
 
-  // codes 8*sub .. 8*sub+7 of this lane's 32, as 8 dequantised 16-bit values
-  __device__ inline typename T::vec8 frag(int j, int sub) const {
-    uint4 d;
+  // code i (0..7) of sub-step `sub` of column tile j, as float
+  __device__ inline float code(int j, int sub, int i, uint32_t even, uint32_t odd) const {
     if constexpr (BITS == 4) {
-      d = dequant8_w4<T>(w[j][0][sub], s[j], b[j]);
+      return ubyte_f32((i & 1) ? odd : even, i >> 1);
     } else {
-      d = dequant8_w8<T>(w[j][sub >> 1][(sub & 1) * 2], w[j][sub >> 1][(sub & 1) * 2 + 1], s[j], b[j]);
+      return ubyte_f32(w[j][sub >> 1][(sub & 1) * 2 + (i >> 2)], i & 3);
     }
-    return __builtin_bit_cast(typename T::vec8, d);
+  }
+  __device__ inline float deq(int j, int sub, int i, uint32_t even, uint32_t odd) const {
+    return __builtin_fmaf(code(j, sub, i, even, odd), s[j], b[j]);
   }
 };
 
@@ -85,8 +91,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int per_xcd = n_tiles / 8;
     if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
   }
-  const int tm = tile % tiles_m;
-  const int tn = tile / tiles_m;
+  // Within an XCD's run, walk the tiles in bands of kBandM tile-rows, row
+  // index fastest: the ~32 workgroups resident on one XCD then cover about
+  // kBandM x 8 tiles and share kBandM x-tiles and 8 weight-tiles per k step.
+  constexpr int kBandM = 4;
+  const int band_tiles = kBandM * tiles_n;
+  const int band = tile / band_tiles;
+  const int band_rows = min(tiles_m - band * kBandM, kBandM);
+  const int in_band = tile - band * band_tiles;
+  const int tm = band * kBandM + in_band % band_rows;
+  const int tn = in_band / band_rows;
   const int m0 = tm * BM;
   const int n0 = tn * BN;
 
@@ -105,81 +119,170 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // this lane's two weight rows (columns of y); rows past N are clamped for loads
-  const uint32_t* wrow[2];
-  const uint16_t* srow[2];
-  const uint16_t* brow[2];
+  // this lane's two weight rows (columns of y); rows past N are clamped for
+  // loads.  Lane half h starts 32 codes into the step; with GS == 32 that is
+  // also one group further.  Byte offsets fit 32 bits (checked by the launcher).
+  uint32_t woff[2], soff[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int n = min(n0 + wn + 32 * j + r, N - 1);
-    wrow[j] = wq + (int64_t)n * (K * BITS / 32);
-    srow[j] = scales + (int64_t)n * (K / GS);
-    brow[j] = biases + (int64_t)n * (K / GS);
+    const uint32_t n = (uint32_t)min(n0 + wn + 32 * j + r, N - 1);
+    woff[j] = n * (uint32_t)(K * BITS / 8) + (uint32_t)(32 * h * BITS / 8);
+    soff[j] = (n * (uint32_t)(K / GS) + (uint32_t)((32 * h) / GS)) * 2u;
   }
   // this thread's share of the x tile: 8 rows, one 16-byte column
-  int xoff[8];  // element offsets; M*K < 2^31 is checked by the launcher
+  uint32_t xoff[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) xoff[i] = min(m0 + (t >> 3) + 32 * i, M - 1) * K + 8 * (t & 7);
+  for (int i = 0; i < 8; ++i) xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+  const char* xbytes = reinterpret_cast<const char*>(x);
+  // LDS addresses: the write slot of this thread (row t/8 of each 32-row block)
+  // and, per k sub-step, the read slot of this lane (row r of each 32-row block)
+  const int wr_slot = swz(t >> 3, t & 7);
+  int rd_slot[4];
+#pragma unroll
+  for (int sub = 0; sub < 4; ++sub) rd_slot[sub] = swz(r, 4 * h + sub);
 
   u32x4 xa[8];
   auto issue_x = [&](int k0) {
+    const char* base = xbytes + (size_t)k0 * 2;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(x + xoff[i] + k0);
+    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(base + xoff[i]);
   };
   auto commit_x = [&](char* tile_x) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(tile_x + swz((t >> 3) + 32 * i, t & 7)) = xa[i];
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(tile_x + wr_slot + 4096 * i) = xa[i];
   };
 
   const int steps = K / BK;
   WeightRegs<T, GS, BITS> wa, wb;
 
-  // One k step: prefetch step+1 (x into registers, weights into `next`), run
-  // the matrix work of `step` from LDS buffer step&1 and `now`, then publish
-  // the prefetched x tile.
-  auto do_step = [&](int step, const WeightRegs<T, GS, BITS>& now, WeightRegs<T, GS, BITS>& next) {
-    const char* xs = lds + (step & 1) * kTileBytes;
-    // branch-free prefetch: the last step re-reads its own operands, which nobody consumes
-    const int k_next = min(step + 1, steps - 1) * BK;
-    issue_x(k_next);
-    next.issue(wrow, srow, brow, k_next, h);
-    // Fragment pipeline over 8 slots (4 k sub-steps x 2 halves of the rows):
-    // the LDS reads of slot q+1 are issued before the matrix work of slot q.
-    vec8 af[2][4];
-    auto read_slot = [&](int q, vec8 (&dst)[4]) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        dst[i] = *reinterpret_cast<const vec8*>(xs + swz(32 * (4 * (q & 1) + i) + r, 4 * h + (q >> 1)));
-    };
-    read_slot(0, af[0]);
-    vec8 b0, b1;
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      if (q < 7) read_slot(q + 1, af[(q + 1) & 1]);
-      if ((q & 1) == 0) {
-        b0 = now.frag(0, q >> 1);
-        b1 = now.frag(1, q >> 1);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        acc[4 * (q & 1) + i][0] = mfma32(af[q & 1][i], b0, acc[4 * (q & 1) + i][0]);
-        acc[4 * (q & 1) + i][1] = mfma32(af[q & 1][i], b1, acc[4 * (q & 1) + i][1]);
-      }
+  // Dequantisation of one 8-code fragment, cut into 7 chunks of at most four
+  // VALU instructions so that a chunk fits in the shadow of one matrix
+  // instruction.  tmp/even/odd carry state between the chunks of a fragment.
+  struct Dq {
+    float tmp[8];
+    uint32_t even, odd;
+  };
+  auto dq_chunk = [&](const WeightRegs<T, GS, BITS>& w, int j, int sub, int c, Dq& d, uint32_t (&out)[4]) {
+    switch (c) {
+      case 0:
+        if constexpr (BITS == 4) {
+          d.even = w.w[j][0][sub] & 0x0f0f0f0fu;
+          d.odd = (w.w[j][0][sub] >> 4) & 0x0f0f0f0fu;
+        }
+        break;
+      case 1:
+        d.tmp[0] = w.deq(j, sub, 0, d.even, d.odd);
+        d.tmp[1] = w.deq(j, sub, 1, d.even, d.odd);
+        break;
+      case 2:
+        out[0] = T::pack2(d.tmp[0], d.tmp[1]);
+        d.tmp[2] = w.deq(j, sub, 2, d.even, d.odd);
+        break;
+      case 3:
+        d.tmp[3] = w.deq(j, sub, 3, d.even, d.odd);
+        out[1] = T::pack2(d.tmp[2], d.tmp[3]);
+        break;
+      case 4:
+        d.tmp[4] = w.deq(j, sub, 4, d.even, d.odd);
+        d.tmp[5] = w.deq(j, sub, 5, d.even, d.odd);
+        break;
+      case 5:
+        out[2] = T::pack2(d.tmp[4], d.tmp[5]);
+        d.tmp[6] = w.deq(j, sub, 6, d.even, d.odd);
+        break;
+      case 6:
+        d.tmp[7] = w.deq(j, sub, 7, d.even, d.odd);
+        out[3] = T::pack2(d.tmp[6], d.tmp[7]);
+        break;
+      default:
+        break;
     }
-    commit_x(lds + ((step + 1) & 1) * kTileBytes);
+  };
+  auto full_frag = [&](const WeightRegs<T, GS, BITS>& w, int j, uint32_t (&out)[4]) {
+    Dq d;
+#pragma unroll
+    for (int c = 0; c < 7; ++c) dq_chunk(w, j, 0, c, d, out);
+  };
+  auto as_frag = [](const uint32_t (&v)[4]) {
+    return __builtin_bit_cast(vec8, make_uint4(v[0], v[1], v[2], v[3]));
+  };
+
+  // One k step, written as 64 groups of (one matrix instruction + its fillers)
+  // in the order they are to issue; a scheduling barrier after every group
+  // keeps that order.  Fillers, per 16-instruction sub-step: the chunks of the
+  // two fragments the NEXT sub-step needs, one LDS read of the next slot's x
+  // fragments after every other matrix instruction, and
+  //   sub-step 0: the global loads of the next step's x tile (one per group),
+  //   sub-step 3: global loads of the weights of step+2 into `now` (whose
+  //               contents were consumed during sub-step 2), then the LDS
+  //               writes that publish the prefetched x tile.
+  // bf carries the fragments of sub-step 0 in and those of the next step out.
+  auto do_step = [&](auto parity, int step, WeightRegs<T, GS, BITS>& now, const WeightRegs<T, GS, BITS>& next,
+                     uint32_t (&bf)[2][4]) {
+    constexpr int kParity = decltype(parity)::value;  // == step & 1, known at compile time
+    const char* xs = lds + kParity * kTileBytes;
+    char* xd = lds + (kParity ^ 1) * kTileBytes;
+    // branch-free prefetch: past the end the last step's operands are re-read and never consumed
+    const int k_x = min(step + 1, steps - 1) * BK;
+    const int k_w = min(step + 2, steps - 1) * BK;
+    vec8 af[2][4];
+    auto read_frag = [&](int q, int i) {
+      af[q & 1][i] = *reinterpret_cast<const vec8*>(xs + rd_slot[q >> 1] + 4096 * (4 * (q & 1) + i));
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) read_frag(0, i);
+    uint32_t nb[2][4];
+    Dq dq;
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      const vec8 b0 = as_frag(bf[0]);
+      const vec8 b1 = as_frag(bf[1]);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) {
+        const int q = 2 * sub + (m >> 3);
+        const int i = (m & 7) >> 1;
+        const int ai = 4 * (q & 1) + i;
+        if (m & 1) {
+          acc[ai][1] = mfma32(af[q & 1][i], b1, acc[ai][1]);
+        } else {
+          acc[ai][0] = mfma32(af[q & 1][i], b0, acc[ai][0]);
+        }
+        // fillers
+        if (sub < 3) {
+          dq_chunk(now, m >> 3, sub + 1, m & 7, dq, nb[m >> 3]);
+        } else {
+          dq_chunk(next, m >> 3, 0, m & 7, dq, nb[m >> 3]);
+        }
+        if ((m & 1) && q < 7) read_frag(q + 1, i);
+        if (sub == 0 && m < 8) xa[m] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k_x * 2 + xoff[m]);
+        if (sub == 3 && m == 0) now.issue(wq, scales, biases, woff, soff, k_w);
+        if (sub == 3 && m >= 8) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m - 8)) = xa[m - 8];
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bf[j][e] = nb[j][e];
+    }
     __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   issue_x(0);
-  wa.issue(wrow, srow, brow, 0, h);
+  wa.issue(wq, scales, biases, woff, soff, 0);
+  wb.issue(wq, scales, biases, woff, soff, min(1, steps - 1) * BK);
   commit_x(lds);
+  uint32_t bf[2][4];
+  full_frag(wa, 0, bf[0]);
+  full_frag(wa, 1, bf[1]);
   __syncthreads();
+  __builtin_amdgcn_sched_barrier(0);
   int step = 0;
   for (; step + 1 < steps; step += 2) {  // straight-line body: two steps with the weight registers swapped
-    do_step(step, wa, wb);
-    do_step(step + 1, wb, wa);
+    do_step(std::integral_constant<int, 0>{}, step, wa, wb, bf);
+    do_step(std::integral_constant<int, 1>{}, step + 1, wb, wa, bf);
   }
-  if (step < steps) do_step(step, wa, wb);
+  if (step < steps) do_step(std::integral_constant<int, 0>{}, step, wa, wb, bf);
 
   // Epilogue: register e of an accumulator is row 8*(e/4) + 4*h + e%4, column r.
 #pragma unroll
@@ -218,7 +321,8 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
       return MFQ_ELAUNCH;
     configured = true;
   }
-  if (M * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;  // 32-bit element offsets into x
+  // 32-bit byte offsets into x, the packed weight and the scales
+  if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, stream,
