@@ -32,7 +32,9 @@ constexpr int BN = 256;
 constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;   // one 16-bit x tile: 32 KiB
-constexpr int kLdsBytes = 2 * kTileBytes; // double buffered
+constexpr int kStageStride = 144;         // bytes per staged output row: 64 16-bit columns + 16 bytes of padding
+constexpr int kStageBytes = 128 * kStageStride;  // one wavefront stages 128 rows of its 64 columns at a time
+constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes;  // double-buffered x tiles + output staging
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -74,65 +76,61 @@ struct WeightRegs {
   }
 };
 
-template <typename T, int GS, int BITS>
+template <typename T, int GS, int BITS, bool kEvenSteps>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
     int N, int K, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
+  using WR = WeightRegs<T, GS, BITS>;
 
-  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
-  // run of tiles so that neighbours in the run (same weight columns, adjacent
-  // x rows) share that XCD's L2.
   const int n_tiles = tiles_m * tiles_n;
-  int tile = blockIdx.x;
-  {
-    const int per_xcd = n_tiles / 8;
-    if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
-  }
-  // Within an XCD's run, walk the tiles in bands of kBandM tile-rows, row
-  // index fastest: the ~32 workgroups resident on one XCD then cover about
-  // kBandM x 8 tiles and share kBandM x-tiles and 8 weight-tiles per k step.
-  constexpr int kBandM = 4;
-  const int band_tiles = kBandM * tiles_n;
-  const int band = tile / band_tiles;
-  const int band_rows = min(tiles_m - band * kBandM, kBandM);
-  const int in_band = tile - band * band_tiles;
-  const int tm = band * kBandM + in_band % band_rows;
-  const int tn = in_band / band_rows;
-  const int m0 = tm * BM;
-  const int n0 = tn * BN;
-
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
   const int wn = wave * 64;
   const int r = lane & 31;
   const int h = lane >> 5;
+  const int steps = K / BK;
 
-  f32x16 acc[8][2];
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  // Persistent workgroups: workgroup b takes tiles b, b + grid, b + 2*grid, ...
+  // Workgroups are dealt round-robin to the 8 XCDs, so with a grid that is a
+  // multiple of 8 a workgroup stays on XCD b%8 and that XCD's workgroups walk
+  // a contiguous run of the tile sequence together.  Inside the run the tiles
+  // are ordered in bands of kBandM tile-rows, row index fastest, so the ~32
+  // tiles in flight on one XCD share kBandM x-tiles and 8 weight-tiles per k
+  // step in that XCD's L2.
+  auto tile_origin = [&](int seq, int& m0, int& n0) {
+    int tile = seq;
+    const int per_xcd = n_tiles / 8;
+    if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
+    constexpr int kBandM = 4;
+    const int band_tiles = kBandM * tiles_n;
+    const int band = tile / band_tiles;
+    const int band_rows = min(tiles_m - band * kBandM, kBandM);
+    const int in_band = tile - band * band_tiles;
+    m0 = (band * kBandM + in_band % band_rows) * BM;
+    n0 = (in_band / band_rows) * BN;
+  };
 
-  // this lane's two weight rows (columns of y); rows past N are clamped for
-  // loads.  Lane half h starts 32 codes into the step; with GS == 32 that is
-  // also one group further.  Byte offsets fit 32 bits (checked by the launcher).
-  uint32_t woff[2], soff[2];
+  // Per-lane byte offsets of the tile the PREFETCH cursor is in (it runs two k
+  // steps ahead of the matrix work and enters the next tile two steps early).
+  // Rows past M / N are clamped for loads.  Lane half h starts 32 codes into a
+  // step; with GS == 32 that is also one group further.  Offsets fit 32 bits
+  // (checked by the launcher).
+  uint32_t woff[2], soff[2], xoff[8];
+  auto set_prefetch_tile = [&](int m0, int n0) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const uint32_t n = (uint32_t)min(n0 + wn + 32 * j + r, N - 1);
-    woff[j] = n * (uint32_t)(K * BITS / 8) + (uint32_t)(32 * h * BITS / 8);
-    soff[j] = (n * (uint32_t)(K / GS) + (uint32_t)((32 * h) / GS)) * 2u;
-  }
-  // this thread's share of the x tile: 8 rows, one 16-byte column
-  uint32_t xoff[8];
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t n = (uint32_t)min(n0 + wn + 32 * j + r, N - 1);
+      woff[j] = n * (uint32_t)(K * BITS / 8) + (uint32_t)(32 * h * BITS / 8);
+      soff[j] = (n * (uint32_t)(K / GS) + (uint32_t)((32 * h) / GS)) * 2u;
+    }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+    for (int i = 0; i < 8; ++i)
+      xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+  };
   const char* xbytes = reinterpret_cast<const char*>(x);
   // LDS addresses: the write slot of this thread (row t/8 of each 32-row block)
   // and, per k sub-step, the read slot of this lane (row r of each 32-row block)
@@ -141,19 +139,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
   for (int sub = 0; sub < 4; ++sub) rd_slot[sub] = swz(r, 4 * h + sub);
 
-  u32x4 xa[8];
-  auto issue_x = [&](int k0) {
-    const char* base = xbytes + (size_t)k0 * 2;
+  // x tile registers: set p receives the tile of a step with parity p, two
+  // steps before it is used, and is published to LDS buffer p one step before.
+  u32x4 xa[2][8];
+  WR wa, wb;            // packed weights of the current even / odd step
+  uint32_t bf[2][4];    // dequantised fragments of the next sub-step to run
+  f32x16 acc[8][2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(base + xoff[i]);
-  };
-  auto commit_x = [&](char* tile_x) {
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(tile_x + wr_slot + 4096 * i) = xa[i];
-  };
-
-  const int steps = K / BK;
-  WeightRegs<T, GS, BITS> wa, wb;
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   // Dequantisation of one 8-code fragment, cut into 7 chunks of at most four
   // VALU instructions so that a chunk fits in the shadow of one matrix
@@ -162,46 +159,52 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     float tmp[8];
     uint32_t even, odd;
   };
-  auto dq_chunk = [&](const WeightRegs<T, GS, BITS>& w, int j, int sub, int c, Dq& d, uint32_t (&out)[4]) {
+  // The empty asm statements pin each chunk where it is written: without them
+  // the optimiser is free to sink the arithmetic to its first use (for the
+  // last sub-step that is the next iteration) and to undo the byte-wise
+  // extraction of the 4-bit codes.
+  auto dq_chunk = [&](const WR& w, int j, int sub, int c, Dq& d, uint32_t (&out)[4]) {
     switch (c) {
       case 0:
         if constexpr (BITS == 4) {
           d.even = w.w[j][0][sub] & 0x0f0f0f0fu;
           d.odd = (w.w[j][0][sub] >> 4) & 0x0f0f0f0fu;
+          asm volatile("" : "+v"(d.even), "+v"(d.odd));
         }
         break;
       case 1:
         d.tmp[0] = w.deq(j, sub, 0, d.even, d.odd);
         d.tmp[1] = w.deq(j, sub, 1, d.even, d.odd);
+        asm volatile("" : "+v"(d.tmp[0]), "+v"(d.tmp[1]));
         break;
       case 2:
         out[0] = T::pack2(d.tmp[0], d.tmp[1]);
         d.tmp[2] = w.deq(j, sub, 2, d.even, d.odd);
+        asm volatile("" : "+v"(out[0]), "+v"(d.tmp[2]));
         break;
       case 3:
         d.tmp[3] = w.deq(j, sub, 3, d.even, d.odd);
         out[1] = T::pack2(d.tmp[2], d.tmp[3]);
+        asm volatile("" : "+v"(out[1]));
         break;
       case 4:
         d.tmp[4] = w.deq(j, sub, 4, d.even, d.odd);
         d.tmp[5] = w.deq(j, sub, 5, d.even, d.odd);
+        asm volatile("" : "+v"(d.tmp[4]), "+v"(d.tmp[5]));
         break;
       case 5:
         out[2] = T::pack2(d.tmp[4], d.tmp[5]);
         d.tmp[6] = w.deq(j, sub, 6, d.even, d.odd);
+        asm volatile("" : "+v"(out[2]), "+v"(d.tmp[6]));
         break;
       case 6:
         d.tmp[7] = w.deq(j, sub, 7, d.even, d.odd);
         out[3] = T::pack2(d.tmp[6], d.tmp[7]);
+        asm volatile("" : "+v"(out[3]));
         break;
       default:
         break;
     }
-  };
-  auto full_frag = [&](const WeightRegs<T, GS, BITS>& w, int j, uint32_t (&out)[4]) {
-    Dq d;
-#pragma unroll
-    for (int c = 0; c < 7; ++c) dq_chunk(w, j, 0, c, d, out);
   };
   auto as_frag = [](const uint32_t (&v)[4]) {
     return __builtin_bit_cast(vec8, make_uint4(v[0], v[1], v[2], v[3]));
@@ -209,22 +212,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   // One k step, written as 64 groups of (one matrix instruction + its fillers)
   // in the order they are to issue; a scheduling barrier after every group
-  // keeps that order.  Fillers, per 16-instruction sub-step: the chunks of the
-  // two fragments the NEXT sub-step needs, one LDS read of the next slot's x
-  // fragments after every other matrix instruction, and
-  //   sub-step 0: the global loads of the next step's x tile (one per group),
-  //   sub-step 3: global loads of the weights of step+2 into `now` (whose
-  //               contents were consumed during sub-step 2), then the LDS
-  //               writes that publish the prefetched x tile.
-  // bf carries the fragments of sub-step 0 in and those of the next step out.
-  auto do_step = [&](auto parity, int step, WeightRegs<T, GS, BITS>& now, const WeightRegs<T, GS, BITS>& next,
-                     uint32_t (&bf)[2][4]) {
-    constexpr int kParity = decltype(parity)::value;  // == step & 1, known at compile time
-    const char* xs = lds + kParity * kTileBytes;
-    char* xd = lds + (kParity ^ 1) * kTileBytes;
-    // branch-free prefetch: past the end the last step's operands are re-read and never consumed
-    const int k_x = min(step + 1, steps - 1) * BK;
-    const int k_w = min(step + 2, steps - 1) * BK;
+  // keeps that order.  `now` / `next` are the weight registers of this step and
+  // the following one; k_pref is the k offset, inside the prefetch cursor's
+  // tile, of the step two ahead.  Fillers, per 16-instruction sub-step: the
+  // chunks of the two fragments the NEXT sub-step needs, one LDS read of the
+  // next slot's x fragments after every other matrix instruction, and
+  //   sub-step 0: global loads of the x tile two steps ahead (one per group),
+  //   sub-step 3: global loads of the weights two steps ahead into `now`
+  //               (consumed during sub-step 2), then the LDS writes that
+  //               publish the x tile of the following step.
+  auto do_step = [&](auto parity, WR& now, const WR& next, int k_pref) {
+    constexpr int kP = decltype(parity)::value;  // parity of the step: LDS buffer and x register set
+    const char* xs = lds + kP * kTileBytes;
+    char* xd = lds + (kP ^ 1) * kTileBytes;
     vec8 af[2][4];
     auto read_frag = [&](int q, int i) {
       af[q & 1][i] = *reinterpret_cast<const vec8*>(xs + rd_slot[q >> 1] + 4096 * (4 * (q & 1) + i));
@@ -243,9 +243,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int i = (m & 7) >> 1;
         const int ai = 4 * (q & 1) + i;
         if (m & 1) {
-          acc[ai][1] = mfma32(af[q & 1][i], b1, acc[ai][1]);
+          acc[ai][1] = mfma32(b1, af[q & 1][i], acc[ai][1]);
         } else {
-          acc[ai][0] = mfma32(af[q & 1][i], b0, acc[ai][0]);
+          acc[ai][0] = mfma32(b0, af[q & 1][i], acc[ai][0]);
         }
         // fillers
         if (sub < 3) {
@@ -254,9 +254,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           dq_chunk(next, m >> 3, 0, m & 7, dq, nb[m >> 3]);
         }
         if ((m & 1) && q < 7) read_frag(q + 1, i);
-        if (sub == 0 && m < 8) xa[m] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k_x * 2 + xoff[m]);
-        if (sub == 3 && m == 0) now.issue(wq, scales, biases, woff, soff, k_w);
-        if (sub == 3 && m >= 8) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m - 8)) = xa[m - 8];
+        if (sub == 0 && m < 8) xa[kP][m] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k_pref * 2 + xoff[m]);
+        if (sub == 3 && m == 0) now.issue(wq, scales, biases, woff, soff, k_pref);
+        if (sub == 3 && m >= 8) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m - 8)) = xa[kP ^ 1][m - 8];
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
@@ -267,53 +267,229 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
   };
+  const std::integral_constant<int, 0> even_step{};
+  const std::integral_constant<int, 1> odd_step{};
 
-  issue_x(0);
-  wa.issue(wq, scales, biases, woff, soff, 0);
-  wb.issue(wq, scales, biases, woff, soff, min(1, steps - 1) * BK);
-  commit_x(lds);
-  uint32_t bf[2][4];
-  full_frag(wa, 0, bf[0]);
-  full_frag(wa, 1, bf[1]);
-  __syncthreads();
-  __builtin_amdgcn_sched_barrier(0);
-  int step = 0;
-  for (; step + 1 < steps; step += 2) {  // straight-line body: two steps with the weight registers swapped
-    do_step(std::integral_constant<int, 0>{}, step, wa, wb, bf);
-    do_step(std::integral_constant<int, 1>{}, step + 1, wb, wa, bf);
-  }
-  if (step < steps) do_step(std::integral_constant<int, 0>{}, step, wa, wb, bf);
+  // Fills the pipeline for the tile the prefetch offsets point at: x(0) into
+  // LDS buffer 0, x(1) into register set 1, weights of steps 0 and 1, and the
+  // fragments of sub-step 0.
+  auto prime = [&]() {
+    const int k1 = min(1, steps - 1) * BK;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[1][i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i]);
+    wa.issue(wq, scales, biases, woff, soff, 0);
+    wb.issue(wq, scales, biases, woff, soff, k1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + wr_slot + 4096 * i) = xa[1][i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[1][i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k1 * 2 + xoff[i]);
+    Dq d;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int c = 0; c < 7; ++c) dq_chunk(wa, j, 0, c, d, bf[j]);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-  // Epilogue: register e of an accumulator is row 8*(e/4) + 4*h + e%4, column r.
+  // Writes the finished tile.  The weights were the matrix instruction's A
+  // operand, so accumulator [ai][j] holds, in register e, output row
+  // m0 + 32*ai + r and column n0 + wn + 32*j + 8*(e/4) + 4*h + e%4: four
+  // consecutive columns per register quad, stored as one 8-byte (16-bit y) or
+  // 16-byte (float32 y) piece.  Nothing waits for the stores; they drain while
+  // the next tile is computed.
+  auto store_tile_direct = [&](int m0, int n0) {
+    int lane_e = lane;  // opaque copy, see store_tile_staged
+    asm volatile("" : "+v"(lane_e));
+    const int r = lane_e & 31;
+    const int h = lane_e >> 5;
+    const bool n_vec_ok = (N & 3) == 0;  // keeps every piece aligned and inside the row
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = n0 + wn + 32 * j + r;
-    if (col >= N) continue;
-    const float bv = bias ? T::to_f32(bias[col]) : 0.f;
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+      for (int eb = 0; eb < 4; ++eb) {
+        const int col = n0 + wn + 32 * j + 8 * eb + 4 * h;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + 32 * i + 8 * (e >> 2) + 4 * h + (e & 3);
-        if (row >= M) continue;
-        const int64_t o = (int64_t)row * N + col;
-        const float v = acc[i][j][e];
-        if (y_is_f32) {
-          reinterpret_cast<float*>(y)[o] = bias ? v + bv : v;
-        } else {
-          uint16_t hv = T::from_f32(v);
-          if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
-          reinterpret_cast<uint16_t*>(y)[o] = hv;
+          for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(col + c, N - 1)]);
+        }
+#pragma unroll
+        for (int ai = 0; ai < 8; ++ai) {
+          const int row = m0 + 32 * ai + r;
+          if (row >= M || col >= N) continue;
+          float v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] = acc[ai][j][4 * eb + c];
+          const int64_t o = (int64_t)row * N + col;
+          if (y_is_f32) {
+            float* dst = reinterpret_cast<float*>(y) + o;
+            if (bias) {
+#pragma unroll
+              for (int c = 0; c < 4; ++c) v[c] += bv[c];
+            }
+            if (n_vec_ok) {
+              *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+              for (int c = 0; c < 4; ++c)
+                if (col + c < N) dst[c] = v[c];
+            }
+          } else {
+            uint16_t hv[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              hv[c] = T::from_f32(v[c]);
+              if (bias) hv[c] = T::from_f32(T::to_f32(hv[c]) + bv[c]);
+            }
+            uint16_t* dst = reinterpret_cast<uint16_t*>(y) + o;
+            if (n_vec_ok) {
+              uint2 pk;
+              pk.x = (uint32_t)hv[0] | ((uint32_t)hv[1] << 16);
+              pk.y = (uint32_t)hv[2] | ((uint32_t)hv[3] << 16);
+              *reinterpret_cast<uint2*>(dst) = pk;
+            } else {
+#pragma unroll
+              for (int c = 0; c < 4; ++c)
+                if (col + c < N) dst[c] = hv[c];
+            }
+          }
         }
       }
     }
+  };
+
+  // 16-bit output with N a multiple of 8: each wavefront transposes its
+  // 256 x 64 block through a private LDS region, 128 rows at a time, so that
+  // every global store instruction writes eight complete 128-byte row
+  // segments (16 bytes per lane).  Rows of the staging region are 144 bytes
+  // apart, which spreads both the 8-byte writes (32 rows at once) and the
+  // 16-byte reads (8 rows at once) over all banks.  The region is private to
+  // the wavefront, so no workgroup barrier is needed.
+  auto store_tile_staged = [&](auto with_bias, int m0, int n0) {
+    constexpr bool kBias = decltype(with_bias)::value;
+    // An opaque copy of the lane id: everything below is derived from it, so
+    // none of this per-tile address arithmetic can be hoisted out of the tile
+    // loop and kept live (spilled) across the k loop.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int r = lane_e & 31;
+    const int h = lane_e >> 5;
+    const int lane = lane_e;
+    char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
+    uint16_t* yout = reinterpret_cast<uint16_t*>(y);
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int eb = 0; eb < 4; ++eb) {
+          const int cl = 32 * j + 8 * eb + 4 * h;  // column inside the wavefront's 64
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (kBias) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(n0 + wn + cl + c, N - 1)]);
+          }
+#pragma unroll
+          for (int a4 = 0; a4 < 4; ++a4) {
+            const int ai = 4 * pass + a4;
+            uint32_t pk[2];
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+              pk[c] = T::pack2(acc[ai][j][4 * eb + 2 * c], acc[ai][j][4 * eb + 2 * c + 1]);
+              if constexpr (kBias)  // second rounding, as a separate add on the 16-bit result would do
+                pk[c] = T::pack2(lo_f32<T>(pk[c]) + bv[2 * c], hi_f32<T>(pk[c]) + bv[2 * c + 1]);
+            }
+            *reinterpret_cast<uint2*>(stage + (32 * a4 + r) * kStageStride + cl * 2) = make_uint2(pk[0], pk[1]);
+          }
+          // keep the compiler from converting the whole tile before the first write
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // read back row-wise: lane l takes 16 bytes (8 columns) of row 8*k + l/8
+      const int cg = n0 + wn + 8 * (lane & 7);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int rl = 8 * k + (lane >> 3);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+        const int row = m0 + 128 * pass + rl;
+        if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
+        if (k & 1) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  auto store_tile = [&](int m0, int n0) {
+    if (!y_is_f32 && (N & 7) == 0) {
+      if (bias) {
+        store_tile_staged(std::true_type{}, m0, n0);
+      } else {
+        store_tile_staged(std::false_type{}, m0, n0);
+      }
+    } else {
+      store_tile_direct(m0, n0);
+    }
+  };
+
+  bool primed = false;
+  for (int seq = blockIdx.x; seq < n_tiles; seq += gridDim.x) {
+    int m0, n0;
+    tile_origin(seq, m0, n0);
+    if (!primed) {
+      set_prefetch_tile(m0, n0);
+      prime();
+    }
+    if constexpr (kEvenSteps) {
+      // straight-line pairs of steps; the prefetch cursor enters the next tile
+      // (if this workgroup has one) for the last pair
+      for (int step = 0; step < steps - 2; step += 2) {
+        do_step(even_step, wa, wb, (step + 2) * BK);
+        do_step(odd_step, wb, wa, (step + 3) * BK);
+      }
+      const bool has_next = seq + (int)gridDim.x < n_tiles;
+      int k_a = (steps - 2) * BK, k_b = (steps - 1) * BK;  // no next tile: re-read the last pair, never consumed
+      if (has_next) {
+        int m1, n1;
+        tile_origin(seq + gridDim.x, m1, n1);
+        set_prefetch_tile(m1, n1);
+        k_a = 0;
+        k_b = BK;
+      }
+      do_step(even_step, wa, wb, k_a);
+      do_step(odd_step, wb, wa, k_b);
+      primed = has_next;
+    } else {
+      int step = 0;
+      for (; step + 1 < steps; step += 2) {
+        do_step(even_step, wa, wb, min(step + 2, steps - 1) * BK);
+        do_step(odd_step, wb, wa, min(step + 3, steps - 1) * BK);
+      }
+      if (step < steps) do_step(even_step, wa, wb, (steps - 1) * BK);
+    }
+    store_tile(m0, n0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   }
 }
 
-template <typename T, int GS, int BITS>
-int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-               const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
-  auto kernel = qmm_kernel<T, GS, BITS>;
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return n;
+}
+
+template <typename T, int GS, int BITS, bool kEvenSteps>
+int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                  const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
+  auto kernel = qmm_kernel<T, GS, BITS, kEvenSteps>;
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -321,14 +497,24 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
       return MFQ_ELAUNCH;
     configured = true;
   }
-  // 32-bit byte offsets into x, the packed weight and the scales
-  if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_m * tiles_n)), dim3(kThreads), kLdsBytes, stream,
-                     (const uint16_t*)x, wq, (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
+  const int n_tiles = tiles_m * tiles_n;
+  const int grid = n_tiles < compute_units() ? n_tiles : compute_units();  // one persistent workgroup per CU
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x, wq,
+                     (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
                      (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n);
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T, int GS, int BITS>
+int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+               const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
+  // 32-bit byte offsets into x, the packed weight and the scales
+  if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
+  if ((K / BK) % 2 == 0)
+    return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
+  return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
 }
 
 template <typename T, int GS>
