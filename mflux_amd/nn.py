@@ -11,6 +11,7 @@ attributes the LoRA wrappers read from a quantized layer
 """
 from __future__ import annotations
 
+import contextlib
 import math
 from typing import Callable
 
@@ -21,6 +22,25 @@ from . import core
 
 def _defaults(group_size: int | None, bits: int | None) -> tuple[int, int]:
     return (64 if group_size is None else group_size, 4 if bits is None else bits)
+
+
+_PLACEHOLDERS = False
+
+
+@contextlib.contextmanager
+def placeholder_quantization():
+    """Inside this context ``to_quantized`` / ``from_linear`` build quantized
+    layers of the right shapes and dtypes with zeroed tensors instead of
+    running the quantize kernel.  For loading stored codes: the reference
+    quantizes the freshly initialised model and then overwrites every packed
+    tensor (src/mflux/models/common/weights/loading/weight_applier.py:45-47);
+    quantizing values that are about to be replaced is skipped here."""
+    global _PLACEHOLDERS
+    previous, _PLACEHOLDERS = _PLACEHOLDERS, True
+    try:
+        yield
+    finally:
+        _PLACEHOLDERS = previous
 
 
 class QuantizedLinear(torch.nn.Module):
@@ -86,7 +106,19 @@ class QuantizedLinear(torch.nn.Module):
         ql = cls.__new__(cls)
         torch.nn.Module.__init__(ql)
         ql.group_size, ql.bits, ql.mode = group_size, bits, mode
-        wq, scales, biases = core.quantize(weight, group_size, bits, mode)
+        if _PLACEHOLDERS:
+            core._check_mode("quantize", mode)
+            core._check_group_bits("quantize", group_size, bits)
+            if input_dims % group_size:
+                raise ValueError(
+                    "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
+                    f"group size {group_size}. However the provided matrix has shape {tuple(weight.shape)}"
+                )
+            wq = torch.zeros((output_dims, input_dims * bits // 32), dtype=torch.uint32, device=weight.device)
+            scales = torch.zeros((output_dims, input_dims // group_size), dtype=weight.dtype, device=weight.device)
+            biases = torch.zeros_like(scales)
+        else:
+            wq, scales, biases = core.quantize(weight, group_size, bits, mode)
         ql.register_buffer("weight", wq)
         ql.register_buffer("scales", scales)
         ql.register_buffer("biases", biases)

@@ -201,6 +201,8 @@ def _storage(dtype: int):
 def c_quantize(w: np.ndarray, dtype: int = BF16, group_size: int = 64, bits: int = 4):
     w = np.ascontiguousarray(w, dtype=_storage(dtype))
     K = w.shape[-1]
+    if w.ndim < 2 or K % group_size:
+        raise ValueError(f"quantize needs ndim >= 2 and a last dimension divisible by {group_size}, got {w.shape}")
     lead = w.shape[:-1]
     wq = np.empty((*lead, K * bits // 32), dtype=np.uint32)
     scales = np.empty((*lead, K // group_size), dtype=_storage(dtype))

@@ -20,11 +20,7 @@ def bf16_bits(x_f32: np.ndarray) -> np.ndarray:
     return o.f32_to_bf16_bits(np.asarray(x_f32, dtype=np.float32))
 
 
-def seeded(config: int, tensor: int, shape, std: float) -> np.ndarray:
-    """Synthetic input convention: numpy default_rng(1000*config + tensor),
-    float32 normal scaled by std."""
-    rng = np.random.default_rng(1000 * config + tensor)
-    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+from cases import seeded  # noqa: E402,F401  (kept importable from conftest)
 
 
 @pytest.fixture(scope="session")

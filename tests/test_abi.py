@@ -1,0 +1,97 @@
+"""The C ABI library loads without a GPU, exports every symbol its header
+declares, and rejects bad arguments with an error code before touching the
+device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mfq.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mfq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_qmm_t"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from mflux_amd import _lib
+
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in include/mfq.h but not exported"
+    # and the binding knows a signature for each of them
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_status_strings():
+    from mflux_amd import _lib
+
+    lib = _lib.load()
+    assert lib.mfq_version() >= 100
+    assert lib.mfq_strerror(0) == b"ok"
+    seen = set()
+    for code in range(-8, 0):
+        msg = lib.mfq_strerror(code)
+        assert msg and msg != b"unknown status"
+        seen.add(msg)
+    assert len(seen) == 8
+    assert lib.mfq_strerror(-99) == b"unknown status"
+
+
+def test_argument_validation_needs_no_device():
+    """Every check runs before the first HIP call, so a caller's mistake is an
+    error code, never a launch."""
+    from mflux_amd import _lib
+
+    lib = _lib.load()
+    E = {"dtype": -1, "group": -2, "bits": -3, "shape": -4, "null": -5, "align": -6}
+    buf = ctypes.create_string_buffer(4096 + 64)
+    base = (ctypes.addressof(buf) + 15) & ~15
+    q = lib.mfq_quantize_affine
+    assert q(base, _lib.BF16, 4, 64, 48, 4, base, base, base, None) == E["group"]
+    assert q(base, _lib.BF16, 4, 64, 64, 5, base, base, base, None) == E["bits"]
+    assert q(base, 7, 4, 64, 64, 4, base, base, base, None) == E["dtype"]
+    assert q(base, _lib.BF16, 4, 96, 64, 4, base, base, base, None) == E["shape"]
+    assert q(base, _lib.BF16, 0, 64, 64, 4, base, base, base, None) == E["shape"]
+    assert q(None, _lib.BF16, 4, 64, 64, 4, base, base, base, None) == E["null"]
+    assert q(base + 2, _lib.BF16, 4, 64, 64, 4, base, base, base, None) == E["align"]
+    d = lib.mfq_dequantize_affine
+    assert d(base, base, base, _lib.BF16, 4, 64, 64, 3, base, _lib.BF16, None) == E["bits"]
+    assert d(base, base, None, _lib.BF16, 4, 64, 64, 4, base, _lib.BF16, None) == E["null"]
+    m = lib.mfq_qmm_t
+    args = dict(x=base, xd=_lib.BF16, M=4, K=128, wq=base, s=base, b=base, sd=_lib.BF16, bias=None, N=8, gs=64,
+                bits=4, y=base, yd=_lib.BF16, stream=None)
+
+    def call(**kw):
+        a = {**args, **kw}
+        return m(a["x"], a["xd"], a["M"], a["K"], a["wq"], a["s"], a["b"], a["sd"], a["bias"], a["N"], a["gs"],
+                 a["bits"], a["y"], a["yd"], a["stream"])
+
+    assert call(xd=_lib.F32) == E["dtype"]          # activations must be 16-bit
+    assert call(sd=_lib.F16) == E["dtype"]          # and of the scales' type
+    assert call(yd=_lib.F16) == E["dtype"]          # output: the scales' type or float32
+    assert call(K=100) == E["shape"]
+    assert call(M=0) == E["shape"]
+    assert call(N=1 << 40) == E["shape"]
+    assert call(wq=None) == E["null"]
+    assert call(x=base + 4) == E["align"]
+    assert call(gs=16) == E["group"]
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from mflux_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmfq.so"))
+    with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
+        _lib.load()

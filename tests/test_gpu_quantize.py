@@ -4,60 +4,9 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import seeded
+from cases import adversarial_groups as _adversarial_groups, seeded, storage as _storage
 
 pytestmark = pytest.mark.gpu
-
-
-def _adversarial_groups(o, n_groups: int, gs: int, seed: int) -> np.ndarray:
-    """float32 rows of groups built to hit the corners of the algorithm:
-    ties at x.5 code boundaries, all-equal groups, zeros of both signs, tiny
-    values under the eps clamp, denormals, a huge dynamic range, max-only and
-    min-only edges."""
-    rng = np.random.default_rng(seed)
-    g = np.empty((n_groups, gs), dtype=np.float32)
-    for i in range(n_groups):
-        kind = i % 12
-        if kind == 0:   # exact grid: codes land on integers and on .5 ties
-            step = np.float32(2.0 ** rng.integers(-12, 4))
-            g[i] = rng.integers(-15, 16, gs).astype(np.float32) * step * np.float32(0.5)
-        elif kind == 1:  # all equal
-            g[i] = np.float32(rng.standard_normal() * 0.02)
-        elif kind == 2:  # zeros of both signs
-            g[i] = np.where(rng.random(gs) < 0.5, np.float32(0.0), np.float32(-0.0))
-        elif kind == 3:  # below the eps clamp
-            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e-8)
-        elif kind == 4:  # float32 denormals (flush to zero in bf16 inputs, kept for f32)
-            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e-40)
-        elif kind == 5:  # huge dynamic range
-            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(10.0) ** rng.integers(-6, 6, gs).astype(np.float32)
-        elif kind == 6:  # all positive: the maximum is the edge
-            g[i] = np.abs(rng.standard_normal(gs)).astype(np.float32)
-        elif kind == 7:  # all negative: the minimum is the edge
-            g[i] = -np.abs(rng.standard_normal(gs)).astype(np.float32)
-        elif kind == 8:  # |min| == |max|
-            v = rng.standard_normal(gs).astype(np.float32)
-            v[0], v[1] = np.float32(-3.0), np.float32(3.0)
-            g[i] = np.clip(v, -3, 3)
-        elif kind == 9:  # one outlier
-            v = rng.standard_normal(gs).astype(np.float32) * np.float32(0.01)
-            v[rng.integers(gs)] = np.float32(50.0)
-            g[i] = v
-        elif kind == 10:  # large magnitudes
-            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(1e30)
-        else:
-            g[i] = rng.standard_normal(gs).astype(np.float32) * np.float32(0.02)
-    return g
-
-
-def _storage(o, f32: np.ndarray, dtype: int) -> np.ndarray:
-    if dtype == o.BF16:
-        return o.f32_to_bf16_bits(f32)
-    if dtype == o.F16:
-        with np.errstate(over="ignore"):
-            h = np.clip(f32, -60000, 60000).astype(np.float16)
-        return h.view(np.uint16)
-    return f32
 
 
 @pytest.mark.parametrize("bits", [4, 8])

@@ -1,0 +1,304 @@
+"""Host logic that needs no device: argument checking of the functional API,
+the module tree walk of nn.quantize, the bit-width policy, and the saved
+directory layout."""
+import json
+
+import pytest
+import torch
+
+import mflux_amd
+from mflux_amd import nn as qnn
+from mflux_amd import weights as W
+
+
+# ---------------------------------------------------------------------------
+# functional API: errors raised before any kernel is reached
+# ---------------------------------------------------------------------------
+def test_quantize_argument_errors():
+    w = torch.zeros(4, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="group size 48 is not supported"):
+        mflux_amd.quantize(w, 48, 4)
+    with pytest.raises(ValueError, match="number of bits 7 is not supported"):
+        mflux_amd.quantize(w, 64, 7)
+    with pytest.raises(ValueError, match="not implemented in this build"):
+        mflux_amd.quantize(w, 64, 3)
+    with pytest.raises(ValueError, match="at least 2 dimension"):
+        mflux_amd.quantize(torch.zeros(128, dtype=torch.bfloat16), 64, 4)
+    with pytest.raises(ValueError, match="divisible by the quantization group size"):
+        mflux_amd.quantize(torch.zeros(4, 96, dtype=torch.bfloat16), 64, 4)
+    with pytest.raises(ValueError, match="floating point"):
+        mflux_amd.quantize(torch.zeros(4, 128, dtype=torch.int32), 64, 4)
+    with pytest.raises(ValueError, match="mode"):
+        mflux_amd.quantize(w, 64, 4, mode="mxfp4")
+
+
+def test_no_cpu_fallback():
+    """A CPU tensor is refused: the kernels are the only implementation."""
+    w = torch.zeros(4, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mflux_amd.quantize(w, 64, 4)
+    wq = torch.zeros(8, 16, dtype=torch.uint32)
+    s = torch.zeros(8, 2, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mflux_amd.quantized_matmul(torch.zeros(2, 128, dtype=torch.bfloat16), wq, s, s)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        mflux_amd.dequantize(wq, s, s)
+
+
+def test_quantized_matmul_shape_errors():
+    wq = torch.zeros(8, 16, dtype=torch.uint32)
+    s = torch.zeros(8, 2, dtype=torch.bfloat16)
+    x = torch.zeros(2, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="should be uint32"):
+        mflux_amd.quantized_matmul(x, wq.to(torch.int32), s, s)
+    with pytest.raises(ValueError, match="same shape"):
+        mflux_amd.quantized_matmul(x, wq, s, s[:, :1])
+    with pytest.raises(ValueError, match="incompatible"):
+        mflux_amd.quantized_matmul(x, wq, s, s, bits=8)
+    with pytest.raises(ValueError, match="does not match"):
+        mflux_amd.quantized_matmul(x[:, :64], wq, s, s)
+
+
+# ---------------------------------------------------------------------------
+# nn.quantize: the tree walk and the predicate protocol
+# ---------------------------------------------------------------------------
+class Attn(torch.nn.Module):
+    def __init__(self, dim):
+        super().__init__()
+        self.to_q = qnn.Linear(dim, dim)
+        self.to_out = torch.nn.ModuleList([qnn.Linear(dim, dim), torch.nn.Identity()])
+        self.norm = torch.nn.LayerNorm(dim)
+
+
+class Net(torch.nn.Module):
+    def __init__(self, dim=128):
+        super().__init__()
+        self.x_embedder = qnn.Linear(96, dim)  # 96 is not a multiple of 64
+        self.blocks = torch.nn.ModuleList([Attn(dim), Attn(dim)])
+        self.proj_out = qnn.Linear(dim, 64, bias=False)
+
+
+def test_tree_walk_paths_and_predicate_arguments():
+    net = Net()
+    seen = []
+
+    def predicate(path, module):
+        seen.append((path, type(module).__name__))
+        return False
+
+    assert qnn.quantize(net, class_predicate=predicate) is net
+    assert [p for p, _ in seen] == [
+        "x_embedder", "blocks.0.to_q", "blocks.0.to_out.0", "blocks.0.to_out.1", "blocks.0.norm",
+        "blocks.1.to_q", "blocks.1.to_out.0", "blocks.1.to_out.1", "blocks.1.norm", "proj_out",
+    ]
+    assert not any(isinstance(m, qnn.QuantizedLinear) for m in net.modules())
+
+
+def test_quantize_replaces_selected_leaves_with_defaults_and_dict_answers():
+    net = Net()
+    calls = {}
+
+    def fake_to_quantized(self, **kw):
+        calls[id(self)] = kw
+        with qnn.placeholder_quantization():
+            return qnn.QuantizedLinear.from_linear(self, **kw)
+
+    import unittest.mock as mock
+
+    def predicate(path, module):
+        if not hasattr(module, "to_quantized"):
+            return False
+        if path == "x_embedder":
+            return False
+        if path == "proj_out":
+            return {"group_size": 32, "bits": 8}
+        return True
+
+    with mock.patch.object(qnn.Linear, "to_quantized", fake_to_quantized):
+        qnn.quantize(net, bits=None, class_predicate=predicate)
+    assert isinstance(net.x_embedder, qnn.Linear)
+    q = net.blocks[1].to_out[0]
+    assert isinstance(q, qnn.QuantizedLinear)
+    assert (q.group_size, q.bits, q.mode) == (64, 4, "affine")           # None -> 64 / 4
+    assert q.weight.dtype == torch.uint32 and tuple(q.weight.shape) == (128, 128 * 4 // 32)
+    assert tuple(q.scales.shape) == tuple(q.biases.shape) == (128, 2)
+    assert q.bias is not None and tuple(q.bias.shape) == (128,)
+    assert (net.proj_out.group_size, net.proj_out.bits) == (32, 8)        # dict answer wins
+    assert net.proj_out.bias is None
+    assert tuple(net.proj_out.weight.shape) == (64, 128 * 8 // 32)
+    assert set(k for kw in calls.values() for k in kw) <= {"group_size", "bits", "mode"}
+    # what a LoRA wrapper reads back from a quantized layer
+    assert q.weight.shape[1] * 32 // q.bits == 128 and q.input_dims == 128 and q.output_dims == 128
+    assert not any(p.requires_grad for p in q.parameters())
+    assert sorted(q.state_dict()) == ["bias", "biases", "scales", "weight"]
+
+
+def test_predicate_true_on_unquantizable_module_raises():
+    net = torch.nn.Sequential(torch.nn.LayerNorm(64))
+    with pytest.raises(ValueError, match="Unable to quantize"):
+        qnn.quantize(net, class_predicate=lambda p, m: True)
+    with pytest.raises(ValueError, match="bool or a dict"):
+        qnn.quantize(Net(), class_predicate=lambda p, m: "yes" if hasattr(m, "to_quantized") else False)
+
+
+def test_default_predicate_hits_group_misaligned_layer():
+    """With the default predicate the 96-wide layer is selected and refused by
+    quantize, which is why model definitions carry shape-aware predicates."""
+    with qnn.placeholder_quantization():
+        with pytest.raises(ValueError, match="divisible by the quantization group size"):
+            qnn.quantize(Net())
+        net = Net()
+        qnn.quantize(net, class_predicate=W.group_aligned_predicate, bits=8)
+    assert isinstance(net.x_embedder, qnn.Linear)
+    assert isinstance(net.proj_out, qnn.QuantizedLinear) and net.proj_out.bits == 8
+
+
+def test_quantized_linear_constructor_on_cpu_is_a_placeholder():
+    q = qnn.QuantizedLinear(256, 64, bias=True, group_size=None, bits=8)
+    assert (q.group_size, q.bits) == (64, 8)
+    assert tuple(q.weight.shape) == (64, 64) and q.weight.dtype == torch.uint32
+    assert "input_dims=256, output_dims=64, bias=True, group_size=64, bits=8" in repr(q)
+    with pytest.raises(ValueError, match="divisible"):
+        qnn.QuantizedLinear(100, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        q(torch.zeros(1, 256, dtype=torch.bfloat16))
+
+
+# ---------------------------------------------------------------------------
+# bit-width policy: every stored x requested combination the reference tests
+# ---------------------------------------------------------------------------
+LEVELS = [None, 3, 4, 5, 6, 8]
+
+
+@pytest.mark.parametrize("stored", LEVELS)
+@pytest.mark.parametrize("requested", LEVELS)
+def test_resolution_table(stored, requested):
+    bits, warning = W.QuantizationResolution.resolve(stored=stored, requested=requested)
+    if stored is None:
+        assert bits == requested and warning is None
+    else:
+        assert bits == stored
+        if requested is None or requested == stored:
+            assert warning is None
+        else:
+            assert f"{stored}-bit" in warning and f"-q {requested}" in warning
+
+
+# ---------------------------------------------------------------------------
+# trees, update, ordering, save / reload
+# ---------------------------------------------------------------------------
+def test_tree_flatten_unflatten_round_trip():
+    t = {"a": {"b": [{"w": 1}, {"w": 2, "v": 3}]}, "c": 4}
+    flat = W.tree_flatten(t)
+    assert flat == [("a.b.0.w", 1), ("a.b.1.w", 2), ("a.b.1.v", 3), ("c", 4)]
+    assert W.tree_unflatten(flat) == t
+
+
+class Definition:
+    @staticmethod
+    def get_components():
+        return [W.ComponentDefinition(name="transformer", hf_subdir="transformer"),
+                W.ComponentDefinition(name="vae", hf_subdir="vae", skip_quantization=True)]
+
+    quantization_predicate = staticmethod(W.group_aligned_predicate)
+
+
+class Pipeline:
+    def __init__(self):
+        self.transformer = Net()
+        self.vae = torch.nn.Sequential(qnn.Linear(64, 64))
+
+
+def _fill_fake_codes(model, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    for m in model.modules():
+        if isinstance(m, qnn.QuantizedLinear):
+            m.weight = torch.randint(0, 2 ** 31 - 1, m.weight.shape, generator=g, dtype=torch.int32).view(torch.uint32)
+            m.scales = torch.randn(m.scales.shape, generator=g).to(m.scales.dtype)
+            m.biases = torch.randn(m.biases.shape, generator=g).to(m.biases.dtype)
+
+
+def test_save_reload_round_trip_and_layout(tmp_path):
+    pipe = Pipeline()
+    pipe.transformer.to(torch.bfloat16)
+    with qnn.placeholder_quantization():
+        qnn.quantize(pipe.transformer, class_predicate=Definition.quantization_predicate, bits=4)
+    _fill_fake_codes(pipe.transformer)
+    W.save_model(pipe, 4, tmp_path, Definition)
+
+    index = json.load(open(tmp_path / "transformer" / "model.safetensors.index.json"))
+    assert index["metadata"] == {"quantization_level": "4", "mflux_version": mflux_amd.__version__}
+    assert set(index["weight_map"].values()) == {"0.safetensors"}
+    assert "blocks.0.to_out.0.scales" in index["weight_map"] and "x_embedder.weight" in index["weight_map"]
+    from safetensors import safe_open
+
+    with safe_open(str(tmp_path / "transformer" / "0.safetensors"), framework="pt") as f:
+        assert f.metadata()["quantization_level"] == "4"
+        assert f.get_slice("blocks.0.to_q.weight").get_dtype() == "U32"
+        assert f.get_slice("blocks.0.to_q.scales").get_dtype() == "BF16"
+        assert f.get_slice("x_embedder.weight").get_dtype() == "BF16"
+
+    tree, level, version = W.try_load_saved_format(tmp_path / "vae")
+    assert level == 4 and version == mflux_amd.__version__
+    assert isinstance(tree, dict) and "0" in tree or isinstance(tree, list)
+
+    # reload into a fresh pipeline: stored level wins over the request, with a warning
+    loaded = W.load_saved(Definition, tmp_path)
+    assert loaded.meta_data.quantization_level == 4
+    fresh = Pipeline()
+    fresh.transformer.to(torch.bfloat16)
+    bits = W.WeightApplier.apply_and_quantize(loaded, {"transformer": fresh.transformer, "vae": fresh.vae}, 8,
+                                              Definition)
+    assert bits == 4
+    a, b = pipe.transformer.state_dict(), fresh.transformer.state_dict()
+    assert list(a) == list(b)
+    for k in a:
+        assert a[k].dtype == b[k].dtype and torch.equal(a[k].view(torch.uint8), b[k].view(torch.uint8)), k
+    assert isinstance(fresh.vae[0], qnn.Linear)  # skip_quantization component stays float
+    assert torch.equal(fresh.vae[0].weight, pipe.vae[0].weight)
+
+
+def test_stored_quantized_component_with_missing_codes_is_refused(tmp_path):
+    pipe = Pipeline()
+    with qnn.placeholder_quantization():
+        qnn.quantize(pipe.transformer, class_predicate=Definition.quantization_predicate, bits=8)
+    sd = {k: v for k, v in pipe.transformer.state_dict().items() if not k.startswith("blocks.1.to_q.")}
+    weights = W.LoadedWeights({"transformer": W.tree_unflatten(list(sd.items()))}, W.MetaData(8, "x"))
+    comp = Definition.get_components()[0]
+    with pytest.raises(ValueError, match="packed tensors are missing"):
+        W.WeightApplier.apply_and_quantize_single(weights, Net(), comp, None, Definition.quantization_predicate)
+    with pytest.raises(ValueError, match="No weights found"):
+        W.WeightApplier.apply_and_quantize_single(W.LoadedWeights({}, W.MetaData()), Net(), comp, None)
+
+
+def test_unquantized_apply_keeps_float_layers():
+    src = Net()
+    weights = W.LoadedWeights({"transformer": W.tree_unflatten(list(src.state_dict().items()))}, W.MetaData())
+    dst = Net()
+    bits = W.WeightApplier.apply_and_quantize(weights, {"transformer": dst}, None, Definition)
+    assert bits is None
+    for (ka, va), (kb, vb) in zip(src.state_dict().items(), dst.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+    assert dst.proj_out.weight.requires_grad
+
+
+def test_split_weights_greedy_order():
+    t = {f"t{i}": torch.zeros(n, dtype=torch.uint8) for i, n in enumerate([60, 50, 30, 200, 10, 10])}
+    shards = W.split_weights(t, max_bytes=100)
+    assert [list(s) for s in shards] == [["t0"], ["t1", "t2"], ["t3"], ["t4", "t5"]]
+    assert W.split_weights({}, 100) == []
+
+
+def test_foreign_directory_is_not_our_format(tmp_path):
+    from safetensors.torch import save_file
+
+    assert W.try_load_saved_format(tmp_path / "nope") == (None, None, None)
+    (tmp_path / "empty").mkdir()
+    assert W.try_load_saved_format(tmp_path / "empty") == (None, None, None)
+    (tmp_path / "hf").mkdir()
+    save_file({"w": torch.zeros(2)}, str(tmp_path / "hf" / "model.safetensors"))
+    assert W.try_load_saved_format(tmp_path / "hf") == (None, None, None)
+    save_file({"w": torch.zeros(2)}, str(tmp_path / "hf" / "model.safetensors"),
+              metadata={"quantization_level": "None", "mflux_version": "0.1"})
+    tree, level, version = W.try_load_saved_format(tmp_path / "hf")
+    assert level is None and version == "0.1" and torch.equal(tree["w"], torch.zeros(2))
