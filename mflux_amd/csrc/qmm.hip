@@ -18,6 +18,11 @@
 //     dequantises a word with one float32 fma per code (single rounding to the
 //     16-bit type) right before the matrix instruction that consumes it.  No
 //     column is dequantised by more than one wavefront.
+//   - scales and biases are read as 8-byte pieces (four consecutive groups of
+//     one weight row) once per "period" of 4*GS/64 k steps and unpacked step by
+//     step.  Reading the 2-byte values one step at a time refetches the same
+//     cache line from L2 for every step of every row, which saturates the L2
+//     and costs a third of the kernel's time.
 //   - the k order inside a step is permuted (lane half h covers k 32h..32h+31)
 //     identically for both operands, which the dot product does not notice.
 #include <type_traits>
@@ -49,15 +54,23 @@ struct WeightRegs {
 
   // woff/soff: this lane's byte offsets of its two weight rows / scale rows;
   // k0 is uniform, so every address is a uniform base plus a 32-bit lane offset.
+  __device__ inline void issue_codes(const uint32_t* wq, const uint32_t (&woff)[2], int k0) {
+    const char* wbase = reinterpret_cast<const char*>(wq) + (size_t)k0 * BITS / 8;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int l = 0; l < kLoads; ++l) w[j][l] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + 16 * l);
+  }
+
+  // codes plus this step's scale and bias, one 2-byte load each (the path for
+  // shapes the period-wise scale loads do not cover)
   __device__ inline void issue(const uint32_t* wq, const uint16_t* scales, const uint16_t* biases,
                                const uint32_t (&woff)[2], const uint32_t (&soff)[2], int k0) {
-    const char* wbase = reinterpret_cast<const char*>(wq) + (size_t)k0 * BITS / 8;
+    issue_codes(wq, woff, k0);
     const char* sbase = reinterpret_cast<const char*>(scales) + (size_t)(k0 / GS) * 2;
     const char* bbase = reinterpret_cast<const char*>(biases) + (size_t)(k0 / GS) * 2;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-#pragma unroll
-      for (int l = 0; l < kLoads; ++l) w[j][l] = *reinterpret_cast<const u32x4*>(wbase + woff[j] + 16 * l);
       s[j] = T::to_f32(*reinterpret_cast<const uint16_t*>(sbase + soff[j]));
       b[j] = T::to_f32(*reinterpret_cast<const uint16_t*>(bbase + soff[j]));
     }
@@ -76,7 +89,40 @@ struct WeightRegs {
   }
 };
 
-template <typename T, int GS, int BITS, bool kEvenSteps>
+// Scales and biases of four consecutive groups of the lane's two weight rows:
+// one period of kPeriod = 4*GS/BK k steps.
+template <typename T, int GS>
+struct ScaleRegs {
+  static constexpr int kPeriod = 4 * GS / BK;  // k steps covered by one load
+  uint2 s[2], b[2];
+
+  // g0: first group of the period (a multiple of 4); soff: byte offsets of the
+  // lane's two scale rows
+  __device__ inline void issue(const uint16_t* scales, const uint16_t* biases, const uint32_t (&soff)[2], int g0) {
+    const char* sbase = reinterpret_cast<const char*>(scales) + (size_t)g0 * 2;
+    const char* bbase = reinterpret_cast<const char*>(biases) + (size_t)g0 * 2;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      s[j] = *reinterpret_cast<const uint2*>(sbase + soff[j]);
+      b[j] = *reinterpret_cast<const uint2*>(bbase + soff[j]);
+    }
+  }
+
+  // Scale and bias of step e (0 <= e < kPeriod) of the period for lane half h.
+  template <typename WR>
+  __device__ inline void extract(WR& dst, int e, int h) const {
+    const int idx = GS >= BK ? e * BK / GS : 2 * e + h;  // group inside the period
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint64_t sv = ((uint64_t)s[j].y << 32) | s[j].x;
+      const uint64_t bv = ((uint64_t)b[j].y << 32) | b[j].x;
+      dst.s[j] = T::to_f32((uint16_t)(sv >> (16 * idx)));
+      dst.b[j] = T::to_f32((uint16_t)(bv >> (16 * idx)));
+    }
+  }
+};
+
+template <typename T, int GS, int BITS, bool kFast>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
@@ -84,6 +130,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   using WR = WeightRegs<T, GS, BITS>;
+  using SR = ScaleRegs<T, GS>;
 
   const int n_tiles = tiles_m * tiles_n;
   const int t = threadIdx.x;
@@ -115,17 +162,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   };
 
   // Per-lane byte offsets of the tile the PREFETCH cursor is in (it runs two k
-  // steps ahead of the matrix work and enters the next tile two steps early).
-  // Rows past M / N are clamped for loads.  Lane half h starts 32 codes into a
-  // step; with GS == 32 that is also one group further.  Offsets fit 32 bits
-  // (checked by the launcher).
+  // steps ahead of the matrix work and enters the next tile two steps early;
+  // the scale cursor runs one period further ahead still).  Rows past M / N are
+  // clamped for loads.  Lane half h starts 32 codes into a step; with GS == 32
+  // that is also one group further (the period-wise loads start at the row's
+  // first group instead and pick the half when unpacking).  Offsets fit 32
+  // bits (checked by the launcher).
   uint32_t woff[2], soff[2], xoff[8];
+  auto set_scale_tile = [&](int n0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint32_t n = (uint32_t)min(n0 + wn + 32 * j + r, N - 1);
+      soff[j] = (n * (uint32_t)(K / GS) + (kFast ? 0u : (uint32_t)((32 * h) / GS))) * 2u;
+    }
+  };
   auto set_prefetch_tile = [&](int m0, int n0) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const uint32_t n = (uint32_t)min(n0 + wn + 32 * j + r, N - 1);
       woff[j] = n * (uint32_t)(K * BITS / 8) + (uint32_t)(32 * h * BITS / 8);
-      soff[j] = (n * (uint32_t)(K / GS) + (uint32_t)((32 * h) / GS)) * 2u;
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -143,6 +198,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // steps before it is used, and is published to LDS buffer p one step before.
   u32x4 xa[2][8];
   WR wa, wb;            // packed weights of the current even / odd step
+  SR sr;                // scales and biases of the period the prefetch cursor is in (kFast only)
   uint32_t bf[2][4];    // dequantised fragments of the next sub-step to run
   f32x16 acc[8][2];
 #pragma unroll
@@ -163,7 +219,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // the optimiser is free to sink the arithmetic to its first use (for the
   // last sub-step that is the next iteration) and to undo the byte-wise
   // extraction of the 4-bit codes.
-  auto dq_chunk = [&](const WR& w, int j, int sub, int c, Dq& d, uint32_t (&out)[4]) {
+  auto dq_chunk = [&](const WR& w, int j, int sub, int c, Dq& d, uint32_t (&out)[4]) __attribute__((always_inline)) {
     switch (c) {
       case 0:
         if constexpr (BITS == 4) {
@@ -221,8 +277,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   //   sub-step 3: global loads of the weights two steps ahead into `now`
   //               (consumed during sub-step 2), then the LDS writes that
   //               publish the x tile of the following step.
-  auto do_step = [&](auto parity, WR& now, const WR& next, int k_pref) {
+  //   kFast: `now` also receives, at that point, the scale and bias of the step
+  //               two ahead (step e_pref of the period held in `sr`); when that
+  //               was the period's last step (`reload`), `sr` is refilled from
+  //               group g_pref on, to be unpacked one step later.
+  auto do_step = [&](auto parity, auto reload, WR& now, const WR& next, int k_pref, int e_pref, int g_pref)
+      __attribute__((always_inline)) {
     constexpr int kP = decltype(parity)::value;  // parity of the step: LDS buffer and x register set
+    constexpr bool kReload = decltype(reload)::value;
     const char* xs = lds + kP * kTileBytes;
     char* xd = lds + (kP ^ 1) * kTileBytes;
     vec8 af[2][4];
@@ -255,7 +317,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         if ((m & 1) && q < 7) read_frag(q + 1, i);
         if (sub == 0 && m < 8) xa[kP][m] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k_pref * 2 + xoff[m]);
-        if (sub == 3 && m == 0) now.issue(wq, scales, biases, woff, soff, k_pref);
+        if (sub == 3 && m == 0) {
+          if constexpr (kFast) {
+            now.issue_codes(wq, woff, k_pref);
+            sr.extract(now, e_pref, h);
+            if constexpr (kReload) sr.issue(scales, biases, soff, g_pref);
+          } else {
+            now.issue(wq, scales, biases, woff, soff, k_pref);
+          }
+        }
         if (sub == 3 && m >= 8) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m - 8)) = xa[kP ^ 1][m - 8];
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -269,6 +339,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   };
   const std::integral_constant<int, 0> even_step{};
   const std::integral_constant<int, 1> odd_step{};
+  const std::false_type keep{};
+  const std::true_type refill{};
 
   // Fills the pipeline for the tile the prefetch offsets point at: x(0) into
   // LDS buffer 0, x(1) into register set 1, weights of steps 0 and 1, and the
@@ -277,8 +349,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int k1 = min(1, steps - 1) * BK;
 #pragma unroll
     for (int i = 0; i < 8; ++i) xa[1][i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i]);
-    wa.issue(wq, scales, biases, woff, soff, 0);
-    wb.issue(wq, scales, biases, woff, soff, k1);
+    if constexpr (kFast) {
+      sr.issue(scales, biases, soff, 0);
+      wa.issue_codes(wq, woff, 0);
+      wb.issue_codes(wq, woff, k1);
+      sr.extract(wa, 0, h);
+      sr.extract(wb, 1, h);
+      if constexpr (SR::kPeriod == 2) sr.issue(scales, biases, soff, 4);  // steps >= 4 here
+    } else {
+      wa.issue(wq, scales, biases, woff, soff, 0);
+      wb.issue(wq, scales, biases, woff, soff, k1);
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + wr_slot + 4096 * i) = xa[1][i];
 #pragma unroll
@@ -435,35 +516,76 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     int m0, n0;
     tile_origin(seq, m0, n0);
     if (!primed) {
+      set_scale_tile(n0);
       set_prefetch_tile(m0, n0);
       prime();
     }
-    if constexpr (kEvenSteps) {
-      // straight-line pairs of steps; the prefetch cursor enters the next tile
-      // (if this workgroup has one) for the last pair
-      for (int step = 0; step < steps - 2; step += 2) {
-        do_step(even_step, wa, wb, (step + 2) * BK);
-        do_step(odd_step, wb, wa, (step + 3) * BK);
-      }
+    if constexpr (kFast) {
+      // Pairs of steps (p, p+1), laid out period by period so that what each
+      // step unpacks is known at compile time.  The odd step of a pair unpacks
+      // the scales of step p+3; when that is the last step of a period it also
+      // refills `sr` with the period of step p+4.  The last period of the tile
+      // is peeled: the scale cursor enters the next tile (if this workgroup has
+      // one) before the pair that refills for it, the code / x cursor before
+      // the last pair.  Without a next tile those prefetches re-read pieces of
+      // this tile and are never consumed.
+      constexpr int kPer = SR::kPeriod;
+      constexpr int kGroupsPerStep2 = 2 * BK / GS;  // groups per step, times two (GS == 128: one)
+      auto pair = [&](auto pos, int k_a, int g) __attribute__((always_inline)) {
+        // pos: position of the pair's even step inside its period
+        constexpr int kPos = decltype(pos)::value;
+        constexpr int e_a = (kPos + 2) % kPer, e_b = (kPos + 3) % kPer;
+        do_step(even_step, keep, wa, wb, k_a, e_a, 0);
+        if constexpr (e_b == kPer - 1) {
+          do_step(odd_step, refill, wb, wa, k_a + BK, e_b, g);
+        } else {
+          do_step(odd_step, keep, wb, wa, k_a + BK, e_b, 0);
+        }
+      };
+      // every pair of a period except its last two
+      auto period_head = [&](int p) __attribute__((always_inline)) {
+        if constexpr (kPer == 8) {
+          pair(std::integral_constant<int, 0>{}, (p + 2) * BK, 0);
+          pair(std::integral_constant<int, 2>{}, (p + 4) * BK, 0);
+        }
+      };
       const bool has_next = seq + (int)gridDim.x < n_tiles;
-      int k_a = (steps - 2) * BK, k_b = (steps - 1) * BK;  // no next tile: re-read the last pair, never consumed
-      if (has_next) {
-        int m1, n1;
-        tile_origin(seq + gridDim.x, m1, n1);
-        set_prefetch_tile(m1, n1);
-        k_a = 0;
-        k_b = BK;
+      for (int p = 0; p < steps - (kPer >= 4 ? kPer : 4); p += kPer) {
+        period_head(p);
+        if constexpr (kPer >= 4) {
+          pair(std::integral_constant<int, kPer - 4>{}, (p + kPer - 2) * BK, (p + kPer) * kGroupsPerStep2 / 2);
+          pair(std::integral_constant<int, kPer - 2>{}, (p + kPer) * BK, 0);
+        } else {
+          pair(std::integral_constant<int, 0>{}, (p + 2) * BK, (p + 4) * kGroupsPerStep2 / 2);
+        }
       }
-      do_step(even_step, wa, wb, k_a);
-      do_step(odd_step, wb, wa, k_b);
+      {
+        const int p = steps - kPer;  // first step of the last period
+        int m1 = m0, n1 = n0;
+        if (has_next) tile_origin(seq + gridDim.x, m1, n1);
+        const int g_last = p * kGroupsPerStep2 / 2;  // this tile's last period, for prefetches nobody consumes
+        if constexpr (kPer >= 4) {
+          period_head(p);
+          if (has_next) set_scale_tile(n1);
+          pair(std::integral_constant<int, kPer - 4>{}, (steps - 2) * BK, has_next ? 0 : g_last);
+          if (has_next) set_prefetch_tile(m1, n1);
+          pair(std::integral_constant<int, kPer - 2>{}, has_next ? 0 : (steps - 2) * BK, 0);
+        } else {
+          // the main loop stopped one period early: steps - 4 and steps - 2 remain
+          if (has_next) set_scale_tile(n1);
+          pair(std::integral_constant<int, 0>{}, (steps - 2) * BK, has_next ? 0 : g_last);
+          if (has_next) set_prefetch_tile(m1, n1);
+          pair(std::integral_constant<int, 0>{}, has_next ? 0 : (steps - 2) * BK, has_next ? 4 : g_last);
+        }
+      }
       primed = has_next;
     } else {
       int step = 0;
       for (; step + 1 < steps; step += 2) {
-        do_step(even_step, wa, wb, min(step + 2, steps - 1) * BK);
-        do_step(odd_step, wb, wa, min(step + 3, steps - 1) * BK);
+        do_step(even_step, keep, wa, wb, min(step + 2, steps - 1) * BK, 0, 0);
+        do_step(odd_step, keep, wb, wa, min(step + 3, steps - 1) * BK, 0, 0);
       }
-      if (step < steps) do_step(even_step, wa, wb, (steps - 1) * BK);
+      if (step < steps) do_step(even_step, keep, wa, wb, (steps - 1) * BK, 0, 0);
     }
     store_tile(m0, n0);
 #pragma unroll
@@ -486,10 +608,10 @@ int compute_units() {
   return n;
 }
 
-template <typename T, int GS, int BITS, bool kEvenSteps>
+template <typename T, int GS, int BITS, bool kFast>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                   const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
-  auto kernel = qmm_kernel<T, GS, BITS, kEvenSteps>;
+  auto kernel = qmm_kernel<T, GS, BITS, kFast>;
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -512,7 +634,12 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
                const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
-  if ((K / BK) % 2 == 0)
+  // period-wise scale loads: whole periods, at least two pairs of steps, and
+  // 8-byte aligned scale rows
+  const int64_t steps = K / BK;
+  constexpr int kPer = ScaleRegs<T, GS>::kPeriod;
+  const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
+  if (steps % kPer == 0 && steps >= 4 && aligned8)
     return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
   return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
 }
