@@ -40,6 +40,7 @@ constexpr int kTileBytes = BM * BK * 2;   // one 16-bit x tile: 32 KiB
 constexpr int kStageStride = 144;         // bytes per staged output row: 64 16-bit columns + 16 bytes of padding
 constexpr int kStageBytes = 128 * kStageStride;  // one wavefront stages 128 rows of its 64 columns at a time
 constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes;  // double-buffered x tiles + output staging
+constexpr int kWriteSub = 2;  // sub-step whose fillers publish the next x tile to LDS
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -274,9 +275,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // chunks of the two fragments the NEXT sub-step needs, one LDS read of the
   // next slot's x fragments after every other matrix instruction, and
   //   sub-step 0: global loads of the x tile two steps ahead (one per group),
+  //   sub-step 2: the LDS writes that publish the x tile of the following step
+  //               (early, so that they have landed when the step's closing
+  //               barrier is reached),
   //   sub-step 3: global loads of the weights two steps ahead into `now`
-  //               (consumed during sub-step 2), then the LDS writes that
-  //               publish the x tile of the following step.
+  //               (consumed during sub-step 2).
   //   kFast: `now` also receives, at that point, the scale and bias of the step
   //               two ahead (step e_pref of the period held in `sr`); when that
   //               was the period's last step (`reload`), `sr` is refilled from
@@ -326,7 +329,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
             now.issue(wq, scales, biases, woff, soff, k_pref);
           }
         }
-        if (sub == 3 && m >= 8) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m - 8)) = xa[kP ^ 1][m - 8];
+        if (sub == kWriteSub && (m & 1) == 0) *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * (m >> 1)) = xa[kP ^ 1][m >> 1];
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll

@@ -3,11 +3,14 @@
 // quantize: bit-identical to MLX's CPU evaluation of mx.quantize(mode="affine")
 // (reached from mflux through nn.quantize,
 // src/mflux/models/common/weights/loading/weight_applier.py:43,46,103).
-// Every lane owns 8 consecutive elements (one 128-bit load for 16-bit
-// types), so a group of GS elements is GS/8 neighbouring lanes of one
-// wavefront; group min/max are butterfly reductions over those lanes.  All
-// float32 operations are the same IEEE operations, in the same order, as the
-// scalar algorithm: true division, round-half-even, no contraction.
+// Two kernels.  16-bit inputs (the weights of every model) use
+// quantize_group_per_lane_kernel, described at its definition.  float32 inputs
+// use quantize_kernel: every lane owns 8 consecutive elements, so a group of GS
+// elements is GS/8 neighbouring lanes of one
+// wavefront; group min/max are butterfly reductions over those lanes (DPP
+// lane moves).  All float32 operations produce the same values, in the same
+// order, as the scalar algorithm: correctly rounded division,
+// round-half-even, no contraction.
 //
 // HBM-bound: 2 bytes read and bits/8 + 4/GS bytes written per element.
 #include "common.h"
@@ -35,6 +38,41 @@ __device__ inline void load8<F32>(const float* w, int64_t chunk, float (&v)[8]) 
   v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
+// ---- exact float32 division with a shared reciprocal ----------------------
+// The compiler's correctly rounded a / d is: scale the operands into a safe
+// range (v_div_scale), r = rcp(d) refined once, a quotient refined twice with
+// fused multiply-adds, undo the scaling (v_div_fmas) and patch special values
+// (v_div_fixup).  When d is a normal number away from the ends of the exponent
+// range, the quotient is not going to be subnormal and a is not tiny, neither
+// operand is scaled and nothing is patched: the result IS the chain of fused
+// multiply-adds below.  A group of 64 elements divides by the same scale 64
+// times, so the reciprocal is computed once and each element costs five
+// operations instead of eleven.
+struct Divisor {
+  float d, r;
+  __device__ inline explicit Divisor(float den) : d(den) {
+    const float r0 = __builtin_amdgcn_rcpf(den);
+    r = __builtin_fmaf(__builtin_fmaf(-den, r0, 1.0f), r0, r0);
+  }
+  __device__ inline float divide(float n) const {
+    float q = n * r;
+    q = __builtin_fmaf(__builtin_fmaf(-d, q, n), r, q);
+    return __builtin_fmaf(__builtin_fmaf(-d, q, n), r, q);
+  }
+};
+
+__device__ inline uint32_t exponent_field(float f) { return (__float_as_uint(f) >> 23) & 0xffu; }
+
+// Lane exchange inside a row of 16 lanes without going through LDS.
+template <int kCtrl>
+__device__ inline float dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xf, 0xf, false));
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <- lane 7-i of its half row
+constexpr int kDppMirror = 0x140;      // lane i <- lane 15-i of its row
+
 template <typename T, int GS, int BITS>
 __global__ __launch_bounds__(256) void quantize_kernel(const typename T::storage* __restrict__ w,
                                                        uint32_t* __restrict__ wq,
@@ -46,6 +84,7 @@ __global__ __launch_bounds__(256) void quantize_kernel(const typename T::storage
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const Divisor by_bins(n_bins);
 
   // The trip count is the same for every lane of a wavefront, and a group is
   // either wholly inside n_chunks or wholly outside, so the cross-lane
@@ -67,35 +106,70 @@ __global__ __launch_bounds__(256) void quantize_kernel(const typename T::storage
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int64_t c = c0 + u * stride;
-      float w_min = v[u][0], w_max = v[u][0];
-#pragma unroll
-      for (int i = 1; i < 8; ++i) {
-        w_min = fminf(w_min, v[u][i]);
-        w_max = fmaxf(w_max, v[u][i]);
+      float w_min = fminf(fminf(v[u][0], v[u][1]), v[u][2]);
+      float w_max = fmaxf(fmaxf(v[u][0], v[u][1]), v[u][2]);
+      w_min = fminf(fminf(w_min, v[u][3]), v[u][4]);
+      w_max = fmaxf(fmaxf(w_max, v[u][3]), v[u][4]);
+      w_min = fminf(fminf(w_min, v[u][5]), fminf(v[u][6], v[u][7]));
+      w_max = fmaxf(fmaxf(w_max, v[u][5]), fmaxf(v[u][6], v[u][7]));
+      w_min = fminf(w_min, dpp<kDppXor1>(w_min));
+      w_max = fmaxf(w_max, dpp<kDppXor1>(w_max));
+      w_min = fminf(w_min, dpp<kDppXor2>(w_min));
+      w_max = fmaxf(w_max, dpp<kDppXor2>(w_max));
+      if constexpr (kLanesPerGroup >= 8) {
+        w_min = fminf(w_min, dpp<kDppHalfMirror>(w_min));
+        w_max = fmaxf(w_max, dpp<kDppHalfMirror>(w_max));
       }
-#pragma unroll
-      for (int off = 1; off < kLanesPerGroup; off <<= 1) {
-        w_min = fminf(w_min, __shfl_xor(w_min, off));
-        w_max = fmaxf(w_max, __shfl_xor(w_max, off));
+      if constexpr (kLanesPerGroup >= 16) {
+        w_min = fminf(w_min, dpp<kDppMirror>(w_min));
+        w_max = fmaxf(w_max, dpp<kDppMirror>(w_max));
       }
       const bool mask = fabsf(w_min) > fabsf(w_max);
-      float scale = (w_max - w_min) / n_bins;
-      scale = (scale < kEps) ? kEps : scale;
-      scale = mask ? scale : -scale;
+      const float range = w_max - w_min;
       const float edge = mask ? w_min : w_max;
-      const float q0 = rintf(edge / scale);
-      float bias = 0.0f;
-      if (q0 != 0.0f) {
-        scale = edge / q0;
-        bias = edge;
-      }
+      // Every division below has a divisor and a dividend well inside the
+      // normal range, and a quotient that is neither huge nor able to round to
+      // a nonzero code while being subnormal, exactly when the range and the
+      // edge are: range in [2^-63, 2^63], edge likewise and within 2^40 of the
+      // range.  (Two distinct floats differ by at least 2^-24 of the larger,
+      // so real data never fails the last test.)
+      const uint32_t er = exponent_field(range), ee = exponent_field(edge);
+      const bool tame = (er - 64u) <= 126u && (ee - 64u) <= 126u && ee <= er + 40u;
+      float scale, bias = 0.0f;
       uint32_t code[8];
+      if (tame) {
+        scale = by_bins.divide(range);
+        scale = (scale < kEps) ? kEps : scale;
+        scale = mask ? scale : -scale;
+        const float q0 = rintf(Divisor(scale).divide(edge));
+        if (q0 != 0.0f) {
+          scale = Divisor(q0).divide(edge);
+          bias = edge;
+        }
+        const Divisor by_scale(scale);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        float q = rintf((v[u][i] - bias) / scale);
-        q = (q < 0.0f) ? 0.0f : q;
-        q = (n_bins < q) ? n_bins : q;
-        code[i] = (uint32_t)q;
+        for (int i = 0; i < 8; ++i) {
+          float q = rintf(by_scale.divide(v[u][i] - bias));
+          q = (q < 0.0f) ? 0.0f : q;
+          q = (n_bins < q) ? n_bins : q;
+          code[i] = (uint32_t)q;
+        }
+      } else {
+        scale = range / n_bins;
+        scale = (scale < kEps) ? kEps : scale;
+        scale = mask ? scale : -scale;
+        const float q0 = rintf(edge / scale);
+        if (q0 != 0.0f) {
+          scale = edge / q0;
+          bias = edge;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float q = rintf((v[u][i] - bias) / scale);
+          q = (q < 0.0f) ? 0.0f : q;
+          q = (n_bins < q) ? n_bins : q;
+          code[i] = (uint32_t)q;
+        }
       }
       if (ok[u]) {
         if constexpr (BITS == 4) {
@@ -114,6 +188,144 @@ __global__ __launch_bounds__(256) void quantize_kernel(const typename T::storage
           biases[c / kLanesPerGroup] = T::from_f32(bias);
         }
       }
+    }
+  }
+}
+
+// 16-bit inputs: one lane quantizes one whole group.
+//
+// A wavefront takes 64 consecutive groups (64 * GS elements, contiguous in
+// memory) per iteration: GS/8 coalesced 128-bit loads per lane, a transpose
+// through a wavefront-private LDS region so that lane l ends up holding group
+// l, then min/max, scale, bias and codes entirely inside the lane.  The
+// per-group work (three divisions, the reciprocal of the scale) is then done
+// once per group instead of once per 8 elements, no cross-lane reduction is
+// needed, and scales/biases leave as 128 contiguous bytes per wavefront.
+// LDS slots are XOR-swizzled so that both the row-wise writes and the
+// group-wise reads touch every bank once per 8 lanes.
+template <int kChunks>
+__device__ inline int stage_slot(int group, int chunk) {
+  const int f = kChunks >= 8 ? (group & 7) : ((group >> 1) & (kChunks - 1));
+  return group * kChunks + (chunk ^ f);
+}
+
+template <typename T, int GS, int BITS>
+__global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint16_t* __restrict__ w,
+                                                                      uint32_t* __restrict__ wq,
+                                                                      uint16_t* __restrict__ scales,
+                                                                      uint16_t* __restrict__ biases,
+                                                                      int64_t n_groups) {
+  constexpr int kChunks = GS / 8;                 // 16-byte pieces per group
+  constexpr int kWordsPerChunk = BITS / 4;        // packed words produced per piece
+  constexpr float n_bins = (float)((1 << BITS) - 1);
+  __shared__ uint4 stage_all[4][kWave * kChunks];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  uint4* stage = stage_all[wave];
+  const uint4* w16 = reinterpret_cast<const uint4*>(w);
+  const int64_t n_chunks = n_groups * kChunks;
+  const int64_t wave_stride = (int64_t)gridDim.x * 4 * kWave;  // groups between a wavefront's iterations
+  const Divisor by_bins(n_bins);
+
+  for (int64_t g0 = ((int64_t)blockIdx.x * 4 + wave) * kWave; g0 < n_groups; g0 += wave_stride) {
+    uint4 raw[kChunks];
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int64_t c = g0 * kChunks + j * kWave + lane;
+      raw[j] = c < n_chunks ? w16[c] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int slot = j * kWave + lane;
+      stage[stage_slot<kChunks>(slot / kChunks, slot % kChunks)] = raw[j];
+    }
+    // the region is private to the wavefront and LDS operations of one
+    // wavefront complete in order, so no barrier is needed
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) raw[i] = stage[stage_slot<kChunks>(lane, i)];
+
+    auto element = [&](int i, int e) -> float {
+      const uint32_t pair = e < 2 ? raw[i].x : e < 4 ? raw[i].y : e < 6 ? raw[i].z : raw[i].w;
+      return (e & 1) ? hi_f32<T>(pair) : lo_f32<T>(pair);
+    };
+    float w_min = element(0, 0), w_max = w_min;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+#pragma unroll
+      for (int e = (i == 0 ? 1 : 0); e < 8; ++e) {
+        const float x = element(i, e);
+        w_min = fminf(w_min, x);
+        w_max = fmaxf(w_max, x);
+      }
+    }
+    const bool mask = fabsf(w_min) > fabsf(w_max);
+    const float range = w_max - w_min;
+    const float edge = mask ? w_min : w_max;
+    const uint32_t er = exponent_field(range), ee = exponent_field(edge);
+    const bool tame = (er - 64u) <= 126u && (ee - 64u) <= 126u && ee <= er + 40u;  // see quantize_kernel
+    float scale, bias = 0.0f;
+    uint32_t words[kChunks * kWordsPerChunk];
+    auto pack = [&](int i, const uint32_t (&code)[8]) {
+      if constexpr (BITS == 4) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) word |= code[e] << (4 * e);
+        words[i] = word;
+      } else {
+        words[2 * i] = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+        words[2 * i + 1] = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+      }
+    };
+    if (tame) {
+      scale = by_bins.divide(range);
+      scale = (scale < kEps) ? kEps : scale;
+      scale = mask ? scale : -scale;
+      const float q0 = rintf(Divisor(scale).divide(edge));
+      if (q0 != 0.0f) {
+        scale = Divisor(q0).divide(edge);
+        bias = edge;
+      }
+      const Divisor by_scale(scale);
+#pragma unroll
+      for (int i = 0; i < kChunks; ++i) {
+        uint32_t code[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float q = rintf(by_scale.divide(element(i, e) - bias));
+          code[e] = (uint32_t)__builtin_amdgcn_fmed3f(q, 0.0f, n_bins);
+        }
+        pack(i, code);
+      }
+    } else {
+      scale = range / n_bins;
+      scale = (scale < kEps) ? kEps : scale;
+      scale = mask ? scale : -scale;
+      const float q0 = rintf(edge / scale);
+      if (q0 != 0.0f) {
+        scale = edge / q0;
+        bias = edge;
+      }
+#pragma unroll
+      for (int i = 0; i < kChunks; ++i) {
+        uint32_t code[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float q = rintf((element(i, e) - bias) / scale);
+          q = (q < 0.0f) ? 0.0f : q;
+          q = (n_bins < q) ? n_bins : q;
+          code[e] = (uint32_t)q;
+        }
+        pack(i, code);
+      }
+    }
+    const int64_t g = g0 + lane;
+    if (g < n_groups) {
+      uint4* out = reinterpret_cast<uint4*>(wq + g * (kChunks * kWordsPerChunk));
+#pragma unroll
+      for (int k = 0; k < kChunks * kWordsPerChunk / 4; ++k)
+        out[k] = make_uint4(words[4 * k], words[4 * k + 1], words[4 * k + 2], words[4 * k + 3]);
+      scales[g] = T::from_f32(scale);
+      biases[g] = T::from_f32(bias);
     }
   }
 }
@@ -169,13 +381,27 @@ template <typename T, int GS>
 int quantize_bits(const void* w, int64_t n_chunks, int bits, uint32_t* wq, void* scales, void* biases,
                   hipStream_t stream) {
   using S = typename T::storage;
-  const int grid = grid_for(n_chunks, kUnroll);
-  if (bits == 4) {
-    hipLaunchKernelGGL((quantize_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
-                       (S*)biases, n_chunks);
+  if constexpr (sizeof(S) == 2) {
+    const int64_t n_groups = n_chunks / (GS / 8);
+    const int64_t blocks = (n_groups + 4 * kWave - 1) / (4 * kWave);  // four wavefronts of 64 groups each
+    const int64_t cap = 256 * 4;  // resident at once on 256 CUs; wavefronts loop over the rest
+    const int grid = (int)(blocks < cap ? blocks : cap);
+    if (bits == 4) {
+      hipLaunchKernelGGL((quantize_group_per_lane_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq,
+                         (S*)scales, (S*)biases, n_groups);
+    } else {
+      hipLaunchKernelGGL((quantize_group_per_lane_kernel<T, GS, 8>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq,
+                         (S*)scales, (S*)biases, n_groups);
+    }
   } else {
-    hipLaunchKernelGGL((quantize_kernel<T, GS, 8>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
-                       (S*)biases, n_chunks);
+    const int grid = grid_for(n_chunks, kUnroll);
+    if (bits == 4) {
+      hipLaunchKernelGGL((quantize_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
+                         (S*)biases, n_chunks);
+    } else {
+      hipLaunchKernelGGL((quantize_kernel<T, GS, 8>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
+                         (S*)biases, n_chunks);
+    }
   }
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }

@@ -119,6 +119,8 @@ int mlxo_quantize(const void* w, int dtype, size_t n_elem, int group_size,
   const int int_per_group = group_size / el_per_int;
   const size_t n_groups = n_elem / (size_t)group_size;
 
+  /* groups are independent; the thread split changes nothing in the results */
+#pragma omp parallel for schedule(static) if (n_groups > 4096)
   for (size_t g = 0; g < n_groups; ++g) {
     const size_t w_idx = g * (size_t)group_size;
     float w_min = MLXO_MIN_INIT;

@@ -99,3 +99,34 @@ def test_quantize_dequantize_error_bound_full_size():
     assert bool((err <= step * (1.0 + 15 * 2.0 ** -9) + 1e-12).all())
     assert float((err <= step * (0.5 + 15 * 2.0 ** -9)).float().mean()) > 0.99
     assert bool((err.amin(dim=2) == 0).all())
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_quantize_bit_exact_wide_exponent_sweep(oracle, bits):
+    """2^25 float32 elements whose groups sweep the exponent range (including
+    the ranges where the kernel switches between its shared-reciprocal division
+    and the compiler's full division) and whose values land on and next to code
+    boundaries: every packed word, scale and bias must equal the oracle's."""
+    import mflux_amd
+    from gpu_util import raw, to_dev
+
+    o = oracle
+    rng = np.random.default_rng(77 + bits)
+    n_groups, gs = 1 << 19, 64
+    n_bins = (1 << bits) - 1
+    expo = rng.integers(-80, 60, size=(n_groups, 1)).astype(np.float32)
+    base = rng.standard_normal((n_groups, gs), dtype=np.float32)
+    # a third of the groups: values placed on exact half-code positions of a power-of-two grid
+    grid = (rng.integers(0, 2 * n_bins + 1, size=(n_groups, gs)).astype(np.float32) * np.float32(0.5)
+            - np.float32(n_bins // 2))
+    kind = rng.integers(0, 3, size=(n_groups, 1))
+    f = np.where(kind == 0, grid, base) * np.exp2(expo)
+    # another third keeps full float32 mantissas; nudge some values by one ulp
+    nudge = rng.integers(-1, 2, size=f.shape).astype(np.int32)
+    f = (f.view(np.int32) + np.where(kind == 2, nudge, 0)).view(np.float32)
+    f = np.where(np.isfinite(f), f, np.float32(0)).astype(np.float32).reshape(1 << 12, -1)
+    exp = o.c_quantize(f, o.F32, gs, bits)
+    got = mflux_amd.quantize(to_dev(f, o.F32), group_size=gs, bits=bits)
+    for what, e, g in zip(("wq", "scales", "biases"), exp, got):
+        bad = np.flatnonzero(raw(g).reshape(-1) != e.reshape(-1))
+        assert bad.size == 0, f"{what}: {bad.size} mismatches, first at {bad[:4]}"
