@@ -6,17 +6,35 @@
 // one or a few activation rows against a wide weight, so the kernel is bound
 // by streaming the packed weight from HBM once.
 //
-// A workgroup of four wavefronts owns 16 output features and walks K in
-// phases.  Every lane streams 128-bit pieces of "its" weight row
-// (row = lane % 16), dequantises them in registers with one float32 fma per
-// code, and feeds them to the 16x16x32 matrix core as the A operand; the B
-// operand is the matching slice of x (column = lane % 16 = activation row,
-// zero beyond M), so all M <= 16 rows come at the cost of one.  The order of k
-// inside the product is permuted consistently for both operands, which a dot
-// product does not notice.  x is staged through LDS one phase ahead and the
-// weight loads of phase p+1 are issued before the arithmetic of phase p, so a
-// wavefront always has two phases of HBM reads in flight.  The four
-// wavefronts split each phase and combine their float32 sums through LDS.
+// Two kernels.
+//
+// qmv_rows_kernel (M <= 4, rows of at most 8 KiB of codes): one wavefront per
+// weight row at a time.  The lanes read the row as consecutive 16-byte pieces
+// (lane l takes piece 64*j + l of the row in load j), i.e. every load
+// instruction covers one contiguous KiB, which is the access pattern that
+// reaches HBM speed; loads of the next row are in flight while the current one
+// is consumed.  Each lane dequantises its own codes (one float32 fma per code,
+// single rounding to the 16-bit type) and owns the matching 8-element slices of
+// x, held in registers for the whole kernel.  The dot products run on the
+// 16x16x32 matrix core with BOTH operands indexed by lane: operand A row i /
+// k-block g is lane i+16g's weights, operand B column j / k-block g is lane
+// j+16g's x slice, so the diagonal D[i][i] is the sum over lanes i, i+16,
+// i+32, i+48 of their private dot products, accumulated over all loads of the
+// row.  The 16 diagonal values are summed across the wavefront when the row
+// ends.  The off-diagonal results are never looked at.
+//
+// qmv_kernel (everything else up to M = 16): a workgroup of four wavefronts
+// owns 16 output features and walks K in phases.  Every lane streams 128-bit
+// pieces of "its" weight row (row = lane % 16), dequantises them in registers,
+// and feeds them to the matrix core as the A operand; the B operand is the
+// matching slice of x (column = lane % 16 = activation row, zero beyond M), so
+// all M <= 16 rows come at the cost of one.  x is staged through LDS one phase
+// ahead and the weight loads of phase p+1 are issued before the arithmetic of
+// phase p.  The four wavefronts split each phase and combine their float32
+// sums through LDS.
+//
+// In both kernels the order of k inside a product is permuted consistently for
+// both operands, which a dot product does not notice.
 #include "common.h"
 
 namespace mfq {
@@ -187,6 +205,292 @@ __global__ __launch_bounds__(256) void qmv_kernel(const uint16_t* __restrict__ x
   }
 }
 
+// ---------------------------------------------------------------------------
+// one wavefront per weight row
+// ---------------------------------------------------------------------------
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <- lane 7-i of its half row
+constexpr int kDppMirror = 0x140;      // lane i <- lane 15-i of its row
+
+template <int kCtrl>
+__device__ inline float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xf, 0xf, false));
+}
+
+// Sum over all 64 lanes, returned in every lane.
+__device__ inline float wave_sum(float v) {
+  v += dpp_f32<kDppXor1>(v);
+  v += dpp_f32<kDppXor2>(v);
+  v += dpp_f32<kDppHalfMirror>(v);
+  v += dpp_f32<kDppMirror>(v);  // every lane now holds the sum of its row of 16
+  const int bits = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+}
+
+template <typename T, int BITS, int kM, int kMaxLoads, bool kCoop>
+struct RowRegs {
+  u32x4 w[kMaxLoads];
+  uint16_t s[kMaxLoads], b[kMaxLoads];  // per-lane loads (when `coop` is off)
+  uint32_t sb;                          // cooperative load: lanes 0..31 hold scale pairs, 32..63 bias pairs
+  uint16_t bias;
+
+  // piece[j]: byte offset of this lane's piece of load j inside a row, or -1
+  // past the end of the row; grp[j]: its group index
+  __device__ inline void issue(const char* wq, const uint16_t* scales, const uint16_t* biases, const uint16_t* bias_v,
+                               int64_t row, int row_bytes, int groups, const int (&piece)[kMaxLoads],
+                               const int (&grp)[kMaxLoads], int lane) {
+    const char* wrow = wq + row * row_bytes;
+    const uint16_t* srow = scales + row * groups;
+    const uint16_t* brow = biases + row * groups;
+    if constexpr (kCoop) {
+      // one load instruction for the whole row's scales and biases (at most 64
+      // groups, an even number): lane i < 32 takes scales 2i, 2i+1, lane 32+i
+      // the biases; consume() hands them to the lanes that need them
+      const int i = lane & 31;
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(lane < 32 ? srow : brow);
+      sb = 2 * i < groups ? src[i] : 0u;
+    } else {
+#pragma unroll
+      for (int j = 0; j < kMaxLoads; ++j) {
+        s[j] = srow[grp[j]];
+        b[j] = brow[grp[j]];
+      }
+    }
+    // codes after the scales: loads return in order, and the first piece cannot
+    // be dequantised before its scale is there
+#pragma unroll
+    for (int j = 0; j < kMaxLoads; ++j) {
+      if (piece[j] >= 0) {
+        w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + piece[j]));
+      } else {
+        w[j] = u32x4{0, 0, 0, 0};
+      }
+    }
+    bias = bias_v ? bias_v[row] : (uint16_t)0;
+  }
+};
+
+template <typename T, int BITS, int kM, int kMaxLoads, bool kCoop>
+__global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq,
+                                                       const uint16_t* __restrict__ scales,
+                                                       const uint16_t* __restrict__ biases,
+                                                       const uint16_t* __restrict__ bias, void* __restrict__ y,
+                                                       int y_is_f32, int M, int N, int K, int gs_shift) {
+  using vec8 = typename T::vec8;
+  using R = RowRegs<T, BITS, kM, kMaxLoads, kCoop>;
+  constexpr int kCodes = 128 / BITS;  // codes in one 16-byte piece
+  constexpr int kSlots = kCodes / 8;  // matrix-core k slots fed by one piece
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row_bytes = K * BITS / 8;
+  const int groups = K >> gs_shift;  // the launcher picked kMaxLoads = ceil(row_bytes / 1024)
+
+  // this lane's pieces: position in the row, group, and its slices of x
+  int piece[kMaxLoads], grp[kMaxLoads];
+  vec8 xf[kM][kMaxLoads][kSlots];
+#pragma unroll
+  for (int j = 0; j < kMaxLoads; ++j) {
+    const int off = (j * kWave + lane) * 16;
+    const bool in_row = off < row_bytes;
+    const int k0 = (j * kWave + lane) * kCodes;
+    piece[j] = in_row ? off : -1;
+    grp[j] = in_row ? (k0 >> gs_shift) : 0;
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+#pragma unroll
+      for (int h = 0; h < kSlots; ++h) {
+        u32x4 v = {0, 0, 0, 0};
+        if (in_row && m < M) v = *reinterpret_cast<const u32x4*>(x + (int64_t)m * K + k0 + 8 * h);
+        xf[m][j][h] = __builtin_bit_cast(vec8, v);
+      }
+    }
+  }
+  // which of the four result registers holds this lane's diagonal element
+  const int diag = (lane & 15) - 4 * (lane >> 4);
+
+  // rows are dealt to wavefronts in contiguous, balanced runs
+  const int64_t n_waves = (int64_t)gridDim.x * (blockDim.x / kWave);
+  const int64_t wave_id = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t row_begin = wave_id * N / n_waves;
+  const int64_t row_end = (wave_id + 1) * N / n_waves;
+  if (row_begin >= row_end) return;
+  const char* wbytes = reinterpret_cast<const char*>(wq);
+
+  auto consume = [&](const R& regs, int64_t row) __attribute__((always_inline)) {
+    f32x4 acc[kM], acc_odd[kM];  // two chains per activation row, so that matrix instructions need not wait for each other
+#pragma unroll
+    for (int m = 0; m < kM; ++m) acc[m] = acc_odd[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < kMaxLoads; ++j) {
+      float sc, bi;
+      if constexpr (kCoop) {
+        const int src = (grp[j] >> 1) * 4;  // byte address of the lane that holds the pair
+        const uint32_t sp = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)regs.sb);
+        const uint32_t bp = (uint32_t)__builtin_amdgcn_ds_bpermute(src + 128, (int)regs.sb);
+        const int sh = (grp[j] & 1) * 16;
+        sc = T::to_f32((uint16_t)(sp >> sh));
+        bi = T::to_f32((uint16_t)(bp >> sh));
+      } else {
+        sc = T::to_f32(regs.s[j]);
+        bi = T::to_f32(regs.b[j]);
+      }
+#pragma unroll
+      for (int h = 0; h < kSlots; ++h) {
+        uint4 wf;
+        if constexpr (BITS == 4) {
+          wf = dequant8_w4<T>(regs.w[j][h], sc, bi);
+        } else {
+          wf = dequant8_w8<T>(regs.w[j][2 * h], regs.w[j][2 * h + 1], sc, bi);
+        }
+#pragma unroll
+        for (int m = 0; m < kM; ++m) {
+          if (kM == 1 && ((j * kSlots + h) & 1)) {
+            acc_odd[m] = mfma16(__builtin_bit_cast(vec8, wf), xf[m][j][h], acc_odd[m]);
+          } else {
+            acc[m] = mfma16(__builtin_bit_cast(vec8, wf), xf[m][j][h], acc[m]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < kM; ++m) {
+      if (kM == 1) acc[m] += acc_odd[m];
+      float v = diag == 0 ? acc[m][0] : diag == 1 ? acc[m][1] : diag == 2 ? acc[m][2] : diag == 3 ? acc[m][3] : 0.f;
+      v = wave_sum(v);
+      if (lane == 0 && m < M) {
+        const int64_t o = (int64_t)m * N + row;
+        if (y_is_f32) {
+          if (bias) v += T::to_f32(regs.bias);
+          reinterpret_cast<float*>(y)[o] = v;
+        } else {
+          uint16_t hv = T::from_f32(v);
+          if (bias) hv = T::from_f32(T::to_f32(hv) + T::to_f32(regs.bias));
+          reinterpret_cast<uint16_t*>(y)[o] = hv;
+        }
+      }
+    }
+  };
+
+  // kDepth rows in flight per wavefront: row r + kDepth - 1 is requested before
+  // row r is consumed
+  constexpr int kDepth = 2;
+  R regs[kDepth];
+#pragma unroll
+  for (int d = 0; d < kDepth - 1; ++d)
+    if (row_begin + d < row_end)
+      regs[d].issue(wbytes, scales, biases, bias, row_begin + d, row_bytes, groups, piece, grp, lane);
+  for (int64_t row = row_begin; row < row_end; row += kDepth) {
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      const int64_t r = row + d;
+      if (r < row_end) {
+        if (r + kDepth - 1 < row_end)
+          regs[(d + kDepth - 1) % kDepth].issue(wbytes, scales, biases, bias, r + kDepth - 1, row_bytes, groups, piece,
+                                                grp, lane);
+        consume(regs[d], r);
+      }
+    }
+  }
+}
+
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return n;
+}
+
+template <typename T, int BITS, int kM, int kMaxLoads, bool kCoop>
+int launch_rows_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                       const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
+  // as many workgroups as are resident at once (the register count of the
+  // instantiation decides), so that every wavefront gets one balanced run of rows
+  auto kernel = qmv_rows_kernel<T, BITS, kM, kMaxLoads, kCoop>;
+  static int blocks_per_cu = 0;
+  if (blocks_per_cu == 0) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) n = 1;
+    blocks_per_cu = n > 4 ? 4 : n;
+  }
+  int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
+  const int64_t max_blocks = (N + 3) / 4;  // at least one row per wavefront
+  if (blocks > max_blocks) blocks = max_blocks;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x, wq,
+                     (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, gs_shift);
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T, int BITS, int kM, int kMaxLoads>
+int launch_rows_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                    const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
+  // a row's scales and biases travel as one cooperative load when they fit it:
+  // at most 64 groups, an even number of them, 4-byte aligned arrays
+  const int64_t groups = K >> gs_shift;
+  const bool coop = groups <= 64 && groups % 2 == 0 &&
+                    ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 3u) == 0;
+  if (coop)
+    return launch_rows_kernel<T, BITS, kM, kMaxLoads, true>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype,
+                                                            stream);
+  return launch_rows_kernel<T, BITS, kM, kMaxLoads, false>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype,
+                                                           stream);
+}
+
+// The kernel is instantiated for the exact number of KiB-sized loads per row:
+// up to 6 for one activation row, up to 3 for two to four (their x slices
+// take four times the registers).
+constexpr int kMaxLoadsOneRow = 6;
+constexpr int kMaxLoadsFourRows = 3;
+
+template <typename T, int BITS, int kM, int kLoads>
+int launch_rows_loads(int64_t n_loads, const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                      const void* biases, const void* bias, int64_t N, int gs_shift, void* y, int y_dtype,
+                      hipStream_t stream) {
+  if (n_loads == kLoads)
+    return launch_rows_one<T, BITS, kM, kLoads>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+  if constexpr (kLoads > 1)
+    return launch_rows_loads<T, BITS, kM, kLoads - 1>(n_loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y,
+                                                      y_dtype, stream);
+  return MFQ_EUNSUPPORTED;
+}
+
+inline int64_t loads_per_row(int64_t K, int bits) { return (K * bits / 8 + 1023) / 1024; }
+
+// One activation row: always (when the row fits the instantiated load counts).
+// Two to four rows: only for short rows; with their x slices in registers the
+// four-row instantiation keeps too few wavefronts resident on long rows and
+// the workgroup-per-16-features kernel is faster there.
+inline bool rows_kernel_covers(int64_t M, int64_t K, int bits) {
+  const int64_t n = loads_per_row(K, bits);
+  return (M == 1 && n <= kMaxLoadsOneRow) || (M <= 4 && n <= 1);
+}
+
+template <typename T>
+int launch_rows(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream) {
+  const int gs_shift = gs == 32 ? 5 : gs == 64 ? 6 : 7;
+  const int64_t n = loads_per_row(K, bits);
+  if (bits == 4) {
+    if (M == 1)
+      return launch_rows_loads<T, 4, 1, kMaxLoadsOneRow>(n, x, M, K, wq, scales, biases, bias, N, gs_shift, y,
+                                                         y_dtype, stream);
+    return launch_rows_loads<T, 4, 4, kMaxLoadsFourRows>(n, x, M, K, wq, scales, biases, bias, N, gs_shift, y,
+                                                         y_dtype, stream);
+  }
+  if (M == 1)
+    return launch_rows_loads<T, 8, 1, kMaxLoadsOneRow>(n, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype,
+                                                       stream);
+  return launch_rows_loads<T, 8, 4, kMaxLoadsFourRows>(n, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype,
+                                                       stream);
+}
+
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
@@ -231,6 +535,12 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream) {
   if (M > kRowsPerBlock) return MFQ_EUNSUPPORTED;
+  if (rows_kernel_covers(M, K, bits)) {
+    if (dtype == MFQ_BF16)
+      return launch_rows<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+    if (dtype == MFQ_F16) return launch_rows<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+    return MFQ_EDTYPE;
+  }
   if (dtype == MFQ_BF16) return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   if (dtype == MFQ_F16) return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   return MFQ_EDTYPE;

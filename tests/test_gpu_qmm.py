@@ -67,6 +67,55 @@ def test_qmv_ragged_shapes(oracle, bits, gs, K, N):
     _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs))
 
 
+@pytest.mark.parametrize("bits,gs,K", [
+    (8, 64, 256), (8, 64, 768), (8, 64, 1024), (8, 64, 1088), (8, 64, 3840), (8, 64, 4096), (8, 64, 5120),
+    (8, 64, 6144), (8, 64, 6208),              # 1..6 loads per row, whole and partial last load; 6208: 7 loads
+    (4, 64, 3072), (4, 64, 3840), (4, 64, 8192), (4, 64, 12288), (4, 64, 15360),
+    (8, 32, 3072), (4, 32, 1024), (4, 32, 96),  # more than 64 groups / odd group count: per-lane scale loads
+    (8, 128, 3072), (4, 128, 2048), (8, 128, 384),
+])
+def test_qmv_single_row_kernel_shapes(oracle, bits, gs, K):
+    """M = 1 over every number of loads per row the one-row kernel is built
+    for, both ways of fetching scales, and the first shape beyond it."""
+    o = oracle
+    N = 203  # not a multiple of the wavefront count: uneven runs of rows
+    args = _case(o, 22, 1, K, N, bits, gs=gs)
+    _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [2, 3, 4])
+def test_qmv_few_rows_short_k(oracle, bits, M):
+    """M = 2..4 with rows of one load: the four-row instantiation, including
+    its zero rows (M = 2, 3) and fewer features than wavefronts."""
+    o = oracle
+    for K, N in ((256, 3072), (768, 50), (1024 if bits == 8 else 2048, 3)):
+        args = _case(o, 23, M, K, N, bits)
+        _assert_close(_run(o, *args, bits), _ref(o, *args, bits))
+
+
+def test_qmv_one_hot_and_float32_output(oracle):
+    """One-hot x through the one-row kernel returns a column of the dequantised
+    weight exactly (float32 output: no rounding beyond the weight's), for every
+    lane position of every load."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    K, N = 3072, 96
+    w = o.f32_to_bf16_bits(seeded(24, 1, (N, K), 0.02))
+    for bits in (4, 8):
+        wq, s, b = o.c_quantize(w, o.BF16, 64, bits)
+        deq = o.bf16_bits_to_f32(o.f32_to_bf16_bits(o.dequantize_exact(wq, s, b, o.BF16, 64, bits).astype(np.float32)))
+        for k in (0, 1, 7, 8, 15, 16, 31, 32, 63, 64, 1023, 1024, 2047, 2048, 3071):
+            xf = np.zeros((1, K), dtype=np.float32)
+            xf[0, k] = 1.0
+            y = mflux_amd.quantized_matmul(to_dev(o.f32_to_bf16_bits(xf), o.BF16).float(), u32_to_dev(wq),
+                                           to_dev(s, o.BF16), to_dev(b, o.BF16), group_size=64, bits=bits)
+            assert y.dtype == torch.float32
+            assert np.array_equal(y.cpu().numpy()[0], deq[:, k]), (bits, k)
+
+
 def test_qmv_adaln_config_full(oracle):
     """BASELINE config 2: SiLU(temb) [M,3072] against W8 [18432,3072]."""
     o = oracle
