@@ -32,6 +32,13 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# L2 <-> fabric bytes per GEMM launch (read + written), mean over the two
+# shapes of the step, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# plain copy of known size; the figures and the commands are in
+# profiles/qmm_w4a16_flux_single_block_m4608.md.  Not measurable from inside
+# this script.
+TRAFFIC_BYTES_PER_LAUNCH = ((569.5e6 + 214.0e6) + (504.8e6 + 35.2e6)) / 2
+
 M_TOKENS = 4608
 LINEARS = (("linear1", 3072, 21504), ("linear2", 15360, 3072))  # (name, K, N)
 GS, BITS = 64, 4
@@ -128,6 +135,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-rows", type=int, default=512)
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the GEMV and quantize measurements (they replay HIP graphs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain 256 MiB device-to-device copy, the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (--gpus 1); nothing is sharded across devices")
@@ -141,6 +153,13 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(3000)
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(7)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- operands of the step, resident in HBM --------------------------------
     ops = []
@@ -156,7 +175,8 @@ def main():
             turn["i"] += 1
             mflux_amd.quantize(copies[turn["i"] % len(copies)], GS, BITS)
 
-        quant_ms[name] = graph_ms(quantize_call, 8, 5, torch)
+        if not args.no_secondary:
+            quant_ms[name] = graph_ms(quantize_call, 8, 5, torch)
         del copies, w
         ops.append((name, x, wq, s, b))
 
@@ -190,7 +210,7 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH,
         "avg_launch_us": round(kernel_ms_per_step * 1e3 / launches, 2),
         "flops_per_launch": flops / launches,
     }
@@ -205,14 +225,14 @@ def main():
     # ---- secondary: W8 GEMV (config 2), cold weights ---------------------------
     gemv = {}
     Kg, Ng = 3072, 18432
-    n_buf = 8
+    n_buf = 0 if args.no_secondary else 8
     bufs = []
     for i in range(n_buf):
         w = (torch.randn(Ng, Kg, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
         bufs.append(mflux_amd.quantize(w, GS, 8))
         del w
     bias = (torch.randn(Ng, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
-    for Mg in (1, 4):
+    for Mg in (() if args.no_secondary else (1, 4)):
         temb = torch.randn(Mg, Kg, device=dev, generator=gen)
         xg = torch.nn.functional.silu(temb).to(torch.bfloat16)
         state = {"i": 0}
@@ -231,7 +251,7 @@ def main():
     del bufs
 
     quant = {}
-    for (name, K, N) in LINEARS:
+    for (name, K, N) in (() if args.no_secondary else LINEARS):
         ms = quant_ms[name]
         nbytes = quantize_bytes(N, K, BITS)
         gbs = nbytes / (ms * 1e-3) / 1e9

@@ -69,7 +69,19 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* 
   if (M <= 16)
     return mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                            (hipStream_t)stream);
-  if (K % 64) return MFQ_EUNSUPPORTED;
+  if (K % 64) {
+    // group size 32 with K an odd multiple of it: the matrix-core GEMM steps k
+    // by 64, so these rare shapes go through the small-M kernel 16 rows at a time
+    const size_t x_row = (size_t)K * 2, y_row = (size_t)N * (y_dtype == MFQ_F32 ? 4 : 2);
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+      const int64_t rows = M - m0 < 16 ? M - m0 : 16;
+      const int rc = mfq::launch_qmv(static_cast<const char*>(x) + m0 * x_row, x_dtype, rows, K, wq, scales, biases,
+                                     bias, N, group_size, bits, static_cast<char*>(y) + m0 * y_row, y_dtype,
+                                     (hipStream_t)stream);
+      if (rc) return rc;
+    }
+    return MFQ_OK;
+  }
   return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                          (hipStream_t)stream);
 }

@@ -137,6 +137,15 @@ def test_qmm_vs_f64(oracle, bits, M, K, N):
     _assert_close(_run(o, *args, bits), _ref(o, *args, bits))
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qmm_k_not_multiple_of_64(oracle, bits):
+    """Group size 32 allows K = 96: large M goes through the small-M kernel in
+    slices of 16 rows (x slices are 16-byte aligned: 96 * 2 * 16 bytes)."""
+    o = oracle
+    args = _case(o, 12, 50, 96, 72, bits, gs=32)
+    _assert_close(_run(o, *args, bits, 32), _ref(o, *args, bits, 32))
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 32), (8, 32), (4, 128), (8, 128)])
 def test_qmm_group_sizes(oracle, bits, gs):
     o = oracle
