@@ -80,6 +80,25 @@ int mfq_dequantize_affine(const uint32_t* wq, const void* scales,
                           int out_dtype, void* stream);
 
 /*
+ * out[i, :] = dequantize(row indices[i] of the packed matrix): the lookup of a
+ * quantized embedding table.  Replaces
+ *   mx.dequantize(weight[x], scales[x], biases[x], group_size, bits)
+ * of MLX's QuantizedEmbedding.__call__, which is what nn.quantize with the
+ * default predicate (src/mflux/models/common/weights/loading/
+ * weight_applier.py:30-31) turns every nn.Embedding into, e.g.
+ * src/mflux/models/flux/model/flux_text_encoder/t5_encoder/t5_encoder.py:11.
+ *   wq      [n_rows, K*bits/32]    uint32
+ *   scales, biases [n_rows, K/group_size]   sb_dtype
+ *   indices [n_indices]            int64 (device); negative values count from
+ *                                  the end; values outside the table are
+ *                                  clamped to its first / last row
+ *   out     [n_indices, K]         out_dtype (sb_dtype or MFQ_F32)
+ */
+int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype,
+                        const int64_t* indices, int64_t n_indices, int64_t n_rows, int64_t K,
+                        int group_size, int bits, void* out, int out_dtype, void* stream);
+
+/*
  * y[m, n] = sum_k x[m, k] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs])
  *           (+ bias[n], added after y has been rounded to y_dtype, which is
  *           what QuantizedLinear.__call__ does with its second op).

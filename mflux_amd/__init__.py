@@ -3,7 +3,7 @@ linears, a drop-in for the MLX operations mflux's diffusion transformers run
 through (``mx.quantize`` / ``nn.quantize`` / ``QuantizedLinear`` /
 ``mx.quantized_matmul``)."""
 from . import nn, weights
-from .core import dequantize, quantize, quantized_matmul
+from .core import dequantize, dequantize_rows, quantize, quantized_matmul
 
-__all__ = ["nn", "weights", "quantize", "dequantize", "quantized_matmul"]
+__all__ = ["nn", "weights", "quantize", "dequantize", "dequantize_rows", "quantized_matmul"]
 __version__ = "0.1.0"

@@ -20,6 +20,7 @@ SIGNATURES = {
     "mfq_strerror": (ctypes.c_char_p, [_INT]),
     "mfq_quantize_affine": (_INT, [_PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _PTR, _PTR, _PTR]),
     "mfq_dequantize_affine": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_dequantize_rows": (_INT, [_PTR, _PTR, _PTR, _INT, _PTR, _I64, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
 }
 

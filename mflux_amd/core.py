@@ -135,6 +135,39 @@ def dequantize(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, grou
     return out
 
 
+def dequantize_rows(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, indices: torch.Tensor,
+                    group_size: int = 64, bits: int = 4, mode: str = "affine",
+                    dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``dequantize(w[indices], scales[indices], biases[indices])`` in one pass:
+    the lookup of a quantized embedding table.  ``indices`` is an integer tensor
+    of any shape; the result has shape ``indices.shape + (K,)``.  Negative
+    indices count from the end; indices outside the table are clamped."""
+    _check_mode("dequantize", mode)
+    _check_group_bits("dequantize", group_size, bits)
+    _check_packed("dequantize", w, scales, biases, group_size, bits)
+    if w.ndim != 2:
+        raise ValueError(f"[dequantize] a table to look rows up in must be 2-D, got shape {tuple(w.shape)}")
+    if indices.dtype.is_floating_point or indices.dtype == torch.bool:
+        raise ValueError(f"[dequantize] indices must be integers, got {indices.dtype}")
+    _require_hip("dequantize", w, "w")
+    out_dtype = scales.dtype if dtype is None else dtype
+    if out_dtype not in (scales.dtype, torch.float32):
+        raise ValueError(f"[dequantize] Output dtype must be {scales.dtype} or float32, got {out_dtype}")
+    K = w.shape[1] * 32 // bits
+    idx = indices.to(device=w.device, dtype=torch.int64).reshape(-1).contiguous()
+    out = torch.empty((idx.numel(), K), dtype=out_dtype, device=w.device)
+    if idx.numel() == 0:
+        return out.reshape(*indices.shape, K)
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    with torch.cuda.device(w.device):
+        rc = _lib.load().mfq_dequantize_rows(
+            w.data_ptr(), scales.data_ptr(), biases.data_ptr(), _DTYPE_CODE[scales.dtype], idx.data_ptr(), idx.numel(),
+            w.shape[0], K, group_size, bits, out.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(w.device),
+        )
+    _lib.check("mfq_dequantize_rows", rc)
+    return out.reshape(*indices.shape, K)
+
+
 def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
                      transpose: bool = True, group_size: int = 64, bits: int = 4, mode: str = "affine",
                      *, bias: torch.Tensor | None = None) -> torch.Tensor:

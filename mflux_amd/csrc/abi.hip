@@ -56,6 +56,19 @@ int mfq_dequantize_affine(const uint32_t* wq, const void* scales, const void* bi
                                 (hipStream_t)stream);
 }
 
+int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype, const int64_t* indices,
+                        int64_t n_indices, int64_t n_rows, int64_t K, int group_size, int bits, void* out,
+                        int out_dtype, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!known(sb_dtype) || !known(out_dtype)) return MFQ_EDTYPE;
+  if (n_indices <= 0 || n_rows <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (n_indices > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!wq || !scales || !biases || !indices || !out) return MFQ_ENULL;
+  if (!mfq::aligned16(wq) || !mfq::aligned16(out)) return MFQ_EALIGN;
+  return mfq::launch_dequantize_rows(wq, scales, biases, sb_dtype, indices, n_indices, n_rows, K, group_size, bits,
+                                     out, out_dtype, (hipStream_t)stream);
+}
+
 int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
               const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
               int y_dtype, void* stream) {

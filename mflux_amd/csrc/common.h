@@ -119,6 +119,9 @@ int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, i
                     void* scales, void* biases, hipStream_t stream);
 int launch_dequantize(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype, int64_t rows,
                       int64_t K, int gs, int bits, void* out, int out_dtype, hipStream_t stream);
+int launch_dequantize_rows(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype,
+                           const int64_t* idx, int64_t n_idx, int64_t n_rows, int64_t K, int gs, int bits, void* out,
+                           int out_dtype, hipStream_t stream);
 int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream);

@@ -371,6 +371,59 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
   }
 }
 
+// Row gather + dequantize: out[i, :] = dequantize(row idx[i] of the packed
+// matrix), the body of a quantized embedding lookup
+// (src/mflux/models/flux/model/flux_text_encoder/t5_encoder/t5_encoder.py:11
+// becomes a QuantizedEmbedding under the default predicate).  One workgroup per
+// looked-up row.  Indices are wrapped once if negative and clamped into
+// [0, n_rows): a bad index reads a valid row instead of faulting.
+template <typename TS, typename TO, int GS, int BITS>
+__global__ __launch_bounds__(256) void dequantize_rows_kernel(const uint32_t* __restrict__ wq,
+                                                              const typename TS::storage* __restrict__ scales,
+                                                              const typename TS::storage* __restrict__ biases,
+                                                              const int64_t* __restrict__ idx, int64_t n_rows,
+                                                              int chunks_per_row,
+                                                              typename TO::storage* __restrict__ out) {
+  constexpr int kLanesPerGroup = GS / 8;
+  int64_t row = idx[blockIdx.x];
+  if (row < 0) row += n_rows;
+  row = row < 0 ? 0 : (row >= n_rows ? n_rows - 1 : row);
+  const int64_t src0 = row * chunks_per_row, dst0 = (int64_t)blockIdx.x * chunks_per_row;
+  for (int c = threadIdx.x; c < chunks_per_row; c += blockDim.x) {
+    const int64_t cs = src0 + c;
+    const float s = TS::to_f32(scales[cs / kLanesPerGroup]);
+    const float b = TS::to_f32(biases[cs / kLanesPerGroup]);
+    float q[8];
+    if constexpr (BITS == 4) {
+      const uint32_t word = wq[cs];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) q[i] = (float)((word >> (4 * i)) & 0xfu);
+    } else {
+      const uint2 words = reinterpret_cast<const uint2*>(wq)[cs];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        q[i] = ubyte_f32(words.x, i);
+        q[4 + i] = ubyte_f32(words.y, i);
+      }
+    }
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = __builtin_fmaf(q[i], s, b);
+    const int64_t cd = dst0 + c;
+    if constexpr (sizeof(typename TO::storage) == 2) {
+      uint4 o;
+      o.x = TO::pack2(r[0], r[1]);
+      o.y = TO::pack2(r[2], r[3]);
+      o.z = TO::pack2(r[4], r[5]);
+      o.w = TO::pack2(r[6], r[7]);
+      reinterpret_cast<uint4*>(out)[cd] = o;
+    } else {
+      reinterpret_cast<float4*>(out)[2 * cd] = make_float4(r[0], r[1], r[2], r[3]);
+      reinterpret_cast<float4*>(out)[2 * cd + 1] = make_float4(r[4], r[5], r[6], r[7]);
+    }
+  }
+}
+
 int grid_for(int64_t n_chunks, int per_thread) {
   const int64_t blocks = (n_chunks + 256LL * per_thread - 1) / (256LL * per_thread);
   const int64_t cap = 256 * 8;  // 8 workgroups per CU keeps ~128 KiB of loads in flight per CU
@@ -442,6 +495,35 @@ int dequantize_gs(const uint32_t* wq, const void* scales, const void* biases, in
   }
 }
 
+template <typename TS, typename TO, int GS>
+int dequantize_rows_bits(const uint32_t* wq, const void* scales, const void* biases, const int64_t* idx, int64_t n_idx,
+                         int64_t n_rows, int chunks_per_row, int bits, void* out, hipStream_t stream) {
+  using SS = typename TS::storage;
+  using SO = typename TO::storage;
+  if (bits == 4) {
+    hipLaunchKernelGGL((dequantize_rows_kernel<TS, TO, GS, 4>), dim3((unsigned)n_idx), dim3(256), 0, stream, wq,
+                       (const SS*)scales, (const SS*)biases, idx, n_rows, chunks_per_row, (SO*)out);
+  } else {
+    hipLaunchKernelGGL((dequantize_rows_kernel<TS, TO, GS, 8>), dim3((unsigned)n_idx), dim3(256), 0, stream, wq,
+                       (const SS*)scales, (const SS*)biases, idx, n_rows, chunks_per_row, (SO*)out);
+  }
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename TS, typename TO>
+int dequantize_rows_gs(const uint32_t* wq, const void* scales, const void* biases, const int64_t* idx, int64_t n_idx,
+                       int64_t n_rows, int chunks_per_row, int gs, int bits, void* out, hipStream_t stream) {
+  switch (gs) {
+    case 32:
+      return dequantize_rows_bits<TS, TO, 32>(wq, scales, biases, idx, n_idx, n_rows, chunks_per_row, bits, out, stream);
+    case 64:
+      return dequantize_rows_bits<TS, TO, 64>(wq, scales, biases, idx, n_idx, n_rows, chunks_per_row, bits, out, stream);
+    default:
+      return dequantize_rows_bits<TS, TO, 128>(wq, scales, biases, idx, n_idx, n_rows, chunks_per_row, bits, out,
+                                               stream);
+  }
+}
+
 }  // namespace
 
 int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, int bits, uint32_t* wq, void* scales,
@@ -468,6 +550,23 @@ int launch_dequantize(const uint32_t* wq, const void* scales, const void* biases
     return dequantize_gs<F16, F32>(wq, scales, biases, n_chunks, gs, bits, out, stream);
   if (sb_dtype == MFQ_F32 && out_dtype == MFQ_F32)
     return dequantize_gs<F32, F32>(wq, scales, biases, n_chunks, gs, bits, out, stream);
+  return MFQ_EUNSUPPORTED;
+}
+
+int launch_dequantize_rows(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype,
+                           const int64_t* idx, int64_t n_idx, int64_t n_rows, int64_t K, int gs, int bits, void* out,
+                           int out_dtype, hipStream_t stream) {
+  const int cpr = (int)(K / 8);
+  if (sb_dtype == MFQ_BF16 && out_dtype == MFQ_BF16)
+    return dequantize_rows_gs<BF16, BF16>(wq, scales, biases, idx, n_idx, n_rows, cpr, gs, bits, out, stream);
+  if (sb_dtype == MFQ_BF16 && out_dtype == MFQ_F32)
+    return dequantize_rows_gs<BF16, F32>(wq, scales, biases, idx, n_idx, n_rows, cpr, gs, bits, out, stream);
+  if (sb_dtype == MFQ_F16 && out_dtype == MFQ_F16)
+    return dequantize_rows_gs<F16, F16>(wq, scales, biases, idx, n_idx, n_rows, cpr, gs, bits, out, stream);
+  if (sb_dtype == MFQ_F16 && out_dtype == MFQ_F32)
+    return dequantize_rows_gs<F16, F32>(wq, scales, biases, idx, n_idx, n_rows, cpr, gs, bits, out, stream);
+  if (sb_dtype == MFQ_F32 && out_dtype == MFQ_F32)
+    return dequantize_rows_gs<F32, F32>(wq, scales, biases, idx, n_idx, n_rows, cpr, gs, bits, out, stream);
   return MFQ_EUNSUPPORTED;
 }
 

@@ -1,4 +1,5 @@
-"""Module-level API: ``quantize``, ``QuantizedLinear``, ``Linear``.
+"""Module-level API: ``quantize``, ``QuantizedLinear``, ``Linear``,
+``QuantizedEmbedding``, ``Embedding``.
 
 Mirrors the part of ``mlx.nn`` that mflux uses to quantize a model and to run
 it: ``nn.quantize(model, class_predicate=..., bits=...)`` at
@@ -136,6 +137,90 @@ class Linear(torch.nn.Linear):
 
     def to_quantized(self, group_size: int | None = None, bits: int | None = None, mode: str = "affine"):
         return QuantizedLinear.from_linear(self, group_size, bits, mode)
+
+
+class QuantizedEmbedding(torch.nn.Module):
+    """Embedding table held as packed codes: ``forward(ids)`` gathers and
+    dequantizes the rows, ``as_linear(x)`` multiplies by the transposed table.
+
+    What MLX's ``nn.Embedding.to_quantized`` produces, and therefore what
+    ``nn.quantize`` with the default predicate turns every embedding into
+    (e.g. src/mflux/models/flux/model/flux_text_encoder/t5_encoder/t5_encoder.py:11).
+    """
+
+    def __init__(self, num_embeddings: int, dims: int, group_size: int | None = None, bits: int | None = None,
+                 mode: str = "affine", *, device=None, dtype: torch.dtype = torch.bfloat16):
+        super().__init__()
+        self.group_size, self.bits = _defaults(group_size, bits)
+        self.mode = mode
+        self.num_embeddings, self.dims = num_embeddings, dims
+        core._check_mode("QuantizedEmbedding", mode)
+        core._check_group_bits("QuantizedEmbedding", self.group_size, self.bits)
+        if dims % self.group_size:
+            raise ValueError(
+                "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
+                f"group size {self.group_size}. However the provided matrix has shape {(num_embeddings, dims)}"
+            )
+        device = torch.device("cpu" if device is None else device)
+        if device.type == "cuda":
+            w = torch.randn((num_embeddings, dims), device=device, dtype=torch.float32) * math.sqrt(1.0 / dims)
+            wq, scales, biases = core.quantize(w.to(dtype), self.group_size, self.bits)
+        else:
+            wq = torch.zeros((num_embeddings, dims * self.bits // 32), dtype=torch.uint32, device=device)
+            scales = torch.zeros((num_embeddings, dims // self.group_size), dtype=dtype, device=device)
+            biases = torch.zeros_like(scales)
+        self.register_buffer("weight", wq)
+        self.register_buffer("scales", scales)
+        self.register_buffer("biases", biases)
+
+    def extra_repr(self) -> str:
+        return f"{self.num_embeddings}, {self.dims}, group_size={self.group_size}, bits={self.bits}, mode={self.mode}"
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return core.dequantize_rows(self.weight, self.scales, self.biases, x, group_size=self.group_size,
+                                    bits=self.bits, mode=self.mode)
+
+    def as_linear(self, x: torch.Tensor) -> torch.Tensor:
+        return core.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
+                                     group_size=self.group_size, bits=self.bits, mode=self.mode)
+
+    @classmethod
+    def from_embedding(cls, embedding_layer: torch.nn.Module, group_size: int | None = None, bits: int | None = None,
+                       mode: str = "affine") -> "QuantizedEmbedding":
+        weight = embedding_layer.weight.detach()
+        num_embeddings, dims = weight.shape
+        group_size, bits = _defaults(group_size, bits)
+        qe = cls.__new__(cls)
+        torch.nn.Module.__init__(qe)
+        qe.group_size, qe.bits, qe.mode = group_size, bits, mode
+        qe.num_embeddings, qe.dims = num_embeddings, dims
+        if _PLACEHOLDERS:
+            core._check_mode("quantize", mode)
+            core._check_group_bits("quantize", group_size, bits)
+            if dims % group_size:
+                raise ValueError(
+                    "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
+                    f"group size {group_size}. However the provided matrix has shape {tuple(weight.shape)}"
+                )
+            wq = torch.zeros((num_embeddings, dims * bits // 32), dtype=torch.uint32, device=weight.device)
+            scales = torch.zeros((num_embeddings, dims // group_size), dtype=weight.dtype, device=weight.device)
+            biases = torch.zeros_like(scales)
+        else:
+            wq, scales, biases = core.quantize(weight, group_size, bits, mode)
+        qe.register_buffer("weight", wq)
+        qe.register_buffer("scales", scales)
+        qe.register_buffer("biases", biases)
+        return qe
+
+
+class Embedding(torch.nn.Embedding):
+    """``torch.nn.Embedding`` with MLX's ``to_quantized`` and ``as_linear``."""
+
+    def as_linear(self, x: torch.Tensor) -> torch.Tensor:
+        return torch.nn.functional.linear(x, self.weight)
+
+    def to_quantized(self, group_size: int | None = None, bits: int | None = None, mode: str = "affine"):
+        return QuantizedEmbedding.from_embedding(self, group_size, bits, mode)
 
 
 def leaf_modules(model: torch.nn.Module):

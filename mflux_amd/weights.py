@@ -171,7 +171,7 @@ def group_aligned_predicate(path: str, module: torch.nn.Module, group_size: int 
 
 
 def _quantized_paths(model: torch.nn.Module) -> list[str]:
-    return [p for p, m in model.named_modules() if isinstance(m, qnn.QuantizedLinear)]
+    return [p for p, m in model.named_modules() if isinstance(m, (qnn.QuantizedLinear, qnn.QuantizedEmbedding))]
 
 
 def _quantize_for_stored(model: torch.nn.Module, predicate: Callable, bits: int) -> list[str]:

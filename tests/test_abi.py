@@ -19,7 +19,8 @@ def declared_functions():
 
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
-    for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_qmm_t"):
+    for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
+                 "mfq_qmm_t"):
         assert must in names
 
 
@@ -68,6 +69,11 @@ def test_argument_validation_needs_no_device():
     d = lib.mfq_dequantize_affine
     assert d(base, base, base, _lib.BF16, 4, 64, 64, 3, base, _lib.BF16, None) == E["bits"]
     assert d(base, base, None, _lib.BF16, 4, 64, 64, 4, base, _lib.BF16, None) == E["null"]
+    g = lib.mfq_dequantize_rows
+    assert g(base, base, base, _lib.BF16, None, 2, 10, 128, 64, 4, base, _lib.BF16, None) == E["null"]
+    assert g(base, base, base, _lib.BF16, base, 0, 10, 128, 64, 4, base, _lib.BF16, None) == E["shape"]
+    assert g(base, base, base, _lib.BF16, base, 2, 10, 100, 64, 4, base, _lib.BF16, None) == E["shape"]
+    assert g(base, base, base, _lib.BF16, base, 2, 10, 128, 64, 6, base, _lib.BF16, None) == E["bits"]
     m = lib.mfq_qmm_t
     args = dict(x=base, xd=_lib.BF16, M=4, K=128, wq=base, s=base, b=base, sd=_lib.BF16, bias=None, N=8, gs=64,
                 bits=4, y=base, yd=_lib.BF16, stream=None)

@@ -130,3 +130,55 @@ def test_quantize_bit_exact_wide_exponent_sweep(oracle, bits):
     for what, e, g in zip(("wq", "scales", "biases"), exp, got):
         bad = np.flatnonzero(raw(g).reshape(-1) != e.reshape(-1))
         assert bad.size == 0, f"{what}: {bad.size} mismatches, first at {bad[:4]}"
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_dequantize_rows_is_gather_then_dequantize(oracle, bits, gs):
+    """The embedding lookup equals dequantize() of the gathered rows, bit for
+    bit, for repeated, negative and out-of-range indices and any index shape."""
+    import mflux_amd
+    from gpu_util import raw, to_dev, u32_to_dev
+
+    o = oracle
+    rows, K = 300, 1024
+    w = o.f32_to_bf16_bits(seeded(9, 60 + bits, (rows, K), 0.05))
+    wq, s, b = o.c_quantize(w, o.BF16, gs, bits)
+    full = o.f32_to_bf16_bits(o.dequantize_exact(wq, s, b, o.BF16, gs, bits).astype(np.float32))
+    idx = np.array([[0, 299, 7, 7], [-1, -300, 150, 3], [1000, -1000, 42, 299]], dtype=np.int64)
+    expect_rows = np.array([[0, 299, 7, 7], [299, 0, 150, 3], [299, 0, 42, 299]])
+    args = (u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16))
+    got = mflux_amd.dequantize_rows(*args, torch.from_numpy(idx).cuda(), group_size=gs, bits=bits)
+    assert tuple(got.shape) == (3, 4, K) and got.dtype == torch.bfloat16
+    assert np.array_equal(raw(got), full[expect_rows])
+    got32 = mflux_amd.dequantize_rows(*args, torch.tensor([5, 6], dtype=torch.int32).cuda(), group_size=gs, bits=bits,
+                                      dtype=torch.float32)
+    assert np.array_equal(raw(got32), o.dequantize_exact(wq, s, b, o.BF16, gs, bits).astype(np.float32)[[5, 6]])
+    empty = mflux_amd.dequantize_rows(*args, torch.zeros((0,), dtype=torch.int64).cuda(), group_size=gs, bits=bits)
+    assert tuple(empty.shape) == (0, K)
+
+
+def test_quantized_embedding_module(oracle):
+    """nn.quantize with the default predicate turns an Embedding into a
+    QuantizedEmbedding whose lookup and as_linear agree with the oracle."""
+    import mflux_amd
+    from gpu_util import raw
+    from mflux_amd import nn as qnn
+
+    o = oracle
+    torch.manual_seed(5)
+    model = torch.nn.Sequential(qnn.Embedding(500, 256)).to(device="cuda", dtype=torch.bfloat16)
+    table = raw(model[0].weight)
+    qnn.quantize(model, bits=8)
+    q = model[0]
+    assert isinstance(q, qnn.QuantizedEmbedding) and (q.bits, q.group_size, q.num_embeddings, q.dims) == (8, 64, 500, 256)
+    wq, s, b = o.c_quantize(table, o.BF16, 64, 8)
+    assert np.array_equal(raw(q.weight), wq) and np.array_equal(raw(q.scales), s) and np.array_equal(raw(q.biases), b)
+    ids = torch.tensor([[1, 2, 3], [499, 0, 2]], device="cuda")
+    full = o.f32_to_bf16_bits(o.dequantize_exact(wq, s, b, o.BF16, 64, 8).astype(np.float32))
+    assert np.array_equal(raw(model(ids)), full[ids.cpu().numpy()])
+    x = torch.randn(3, 256, device="cuda").to(torch.bfloat16)
+    y = q.as_linear(x)
+    ref = o.quantized_matmul_f64(x.double().cpu().numpy(), wq, s, b, o.BF16, 64, 8)
+    err = np.abs(y.double().cpu().numpy() - ref).max(axis=1) / np.abs(ref).max(axis=1)
+    assert tuple(y.shape) == (3, 500) and err.max() <= 1e-2

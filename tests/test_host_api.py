@@ -153,6 +153,23 @@ def test_default_predicate_hits_group_misaligned_layer():
     assert isinstance(net.proj_out, qnn.QuantizedLinear) and net.proj_out.bits == 8
 
 
+def test_embedding_is_quantizable_and_walked():
+    model = torch.nn.ModuleDict({"shared": qnn.Embedding(100, 128), "proj": qnn.Linear(128, 64)})
+    with qnn.placeholder_quantization():
+        qnn.quantize(model, bits=8)
+    e = model["shared"]
+    assert isinstance(e, qnn.QuantizedEmbedding) and isinstance(model["proj"], qnn.QuantizedLinear)
+    assert (e.num_embeddings, e.dims, e.bits, e.group_size) == (100, 128, 8, 64)
+    assert tuple(e.weight.shape) == (100, 32) and tuple(e.scales.shape) == (100, 2)
+    assert sorted(e.state_dict()) == ["biases", "scales", "weight"]
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        e(torch.tensor([1, 2]))
+    with pytest.raises(ValueError, match="divisible"):
+        qnn.QuantizedEmbedding(10, 96)
+    plain = qnn.Embedding(10, 64)
+    assert torch.equal(plain.as_linear(torch.ones(1, 64)), torch.ones(1, 64) @ plain.weight.T)
+
+
 def test_quantized_linear_constructor_on_cpu_is_a_placeholder():
     q = qnn.QuantizedLinear(256, 64, bias=True, group_size=None, bits=8)
     assert (q.group_size, q.bits) == (64, 8)
