@@ -18,10 +18,15 @@
  *   - the return value is MFQ_OK (0) or a negative MFQ_E* code; nothing is
  *     thrown across the boundary and nothing is launched when an error is
  *     returned.  mfq_strerror() names a code.
- *   - packed layout (identical to MLX's): element i of a row is the
- *     `bits`-wide field at bit offset (i % (32/bits)) * bits of the uint32
- *     word i / (32/bits); scales and biases hold one value per `group_size`
+ *   - packed layout (identical to MLX's): a row's codes form one little-endian
+ *     bit stream, element i in bits [i*bits, (i+1)*bits).  For 4 and 8 bits
+ *     that is the field at bit offset (i % (32/bits)) * bits of the uint32
+ *     word i / (32/bits); for 3, 5 and 6 bits it is MLX's 3- and 5-byte packs
+ *     laid end to end.  scales and biases hold one value per `group_size`
  *     consecutive elements of a row.
+ *   - bits: 3, 4, 5, 6, 8 for quantize / dequantize / dequantize_rows (3, 5, 6
+ *     for 16-bit inputs only); 4 and 8 for qmm_t (MFQ_EUNSUPPORTED otherwise:
+ *     dequantize and use a plain GEMM).
  */
 #ifndef MFQ_H
 #define MFQ_H
@@ -39,7 +44,7 @@ enum mfq_status {
   MFQ_OK = 0,
   MFQ_EDTYPE = -1,     /* unknown or unsupported dtype code                  */
   MFQ_EGROUP = -2,     /* group_size not in {32, 64, 128}                    */
-  MFQ_EBITS = -3,      /* bits not in {4, 8}                                 */
+  MFQ_EBITS = -3,      /* bits not in {3, 4, 5, 6, 8}                        */
   MFQ_ESHAPE = -4,     /* K not a multiple of group_size, or a size <= 0     */
   MFQ_ENULL = -5,      /* a required pointer is NULL                         */
   MFQ_EALIGN = -6,     /* a buffer is not 16-byte aligned                    */

@@ -19,7 +19,8 @@ from . import _lib
 _DTYPE_CODE = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
 SUPPORTED_GROUP_SIZES = (32, 64, 128)
 MLX_BITS = (2, 3, 4, 5, 6, 8)  # what mx.quantize accepts
-SUPPORTED_BITS = (4, 8)  # what this build has kernels for
+SUPPORTED_BITS = (3, 4, 5, 6, 8)  # what quantize / dequantize have kernels for
+MATMUL_KERNEL_BITS = (4, 8)  # what the matvec / GEMM kernels unpack themselves
 
 
 def _stream_ptr(device: torch.device) -> int:
@@ -43,7 +44,7 @@ def _check_group_bits(fn: str, group_size: int, bits: int) -> None:
             "The supported bits are 2, 3, 4, 5, 6 and 8."
         )
     if bits not in SUPPORTED_BITS:
-        raise ValueError(f"[{fn}] {bits}-bit packing is not implemented in this build (4 and 8 are).")
+        raise ValueError(f"[{fn}] {bits}-bit packing is not implemented in this build (3, 4, 5, 6 and 8 are).")
 
 
 def _require_hip(fn: str, t: torch.Tensor, name: str) -> None:
@@ -75,6 +76,9 @@ def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4, mode: str = "
             "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
             f"group size {group_size}. However the provided matrix has shape {tuple(w.shape)}"
         )
+    if bits not in MATMUL_KERNEL_BITS and w.dtype == torch.float32:
+        raise NotImplementedError(f"[quantize] {bits}-bit quantization of float32 input is not implemented in "
+                                  "this build; cast to bfloat16 or float16")
     _require_hip("quantize", w, "w")
     w = w.contiguous()
     lead = tuple(w.shape[:-1])
@@ -218,6 +222,16 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
             raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
         bias = bias.to(compute).contiguous()
     w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    if bits not in MATMUL_KERNEL_BITS:
+        # 3, 5 and 6 bits: the matmul kernels do not unpack these widths.  The
+        # weight is dequantized by this library's kernel (same single rounding
+        # as inside the fused kernels) and multiplied by the BLAS library's
+        # plain GEMM, float32 accumulation; the bias is added after rounding y.
+        w_full = dequantize(w, scales, biases, group_size, bits)
+        y = torch.matmul(x2, w_full.t()) if out_dtype == compute else torch.matmul(x2.float(), w_full.float().t())
+        if bias is not None:
+            y = y + bias.to(y.dtype)
+        return y.reshape(*lead, N)
     with torch.cuda.device(x.device):
         rc = _lib.load().mfq_qmm_t(
             x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),

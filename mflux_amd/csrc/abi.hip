@@ -7,7 +7,7 @@ namespace {
 
 int check_common(int gs, int bits) {
   if (gs != 32 && gs != 64 && gs != 128) return MFQ_EGROUP;
-  if (bits != 4 && bits != 8) return MFQ_EBITS;
+  if (bits != 3 && bits != 4 && bits != 5 && bits != 6 && bits != 8) return MFQ_EBITS;
   return MFQ_OK;
 }
 
@@ -25,7 +25,7 @@ const char* mfq_strerror(int status) {
     case MFQ_OK: return "ok";
     case MFQ_EDTYPE: return "unsupported dtype";
     case MFQ_EGROUP: return "group_size must be 32, 64 or 128";
-    case MFQ_EBITS: return "bits must be 4 or 8";
+    case MFQ_EBITS: return "bits must be 3, 4, 5, 6 or 8";
     case MFQ_ESHAPE: return "bad shape: sizes must be positive and K a multiple of group_size";
     case MFQ_ENULL: return "null pointer";
     case MFQ_EALIGN: return "buffers must be 16-byte aligned";
@@ -73,6 +73,7 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* 
               const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
               int y_dtype, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
+  if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;  // 3, 5, 6 bits: dequantize, then a plain GEMM
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
   if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;

@@ -279,7 +279,8 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
                                                        const uint16_t* __restrict__ scales,
                                                        const uint16_t* __restrict__ biases,
                                                        const uint16_t* __restrict__ bias, void* __restrict__ y,
-                                                       int y_is_f32, int M, int N, int K, int gs_shift) {
+                                                       int y_is_f32, int M, int N, int K, int gs_shift, int rows_per_wave,
+                                                       int extra_rows) {
   using vec8 = typename T::vec8;
   using R = RowRegs<T, BITS, kM, kMaxLoads, kCoop>;
   constexpr int kCodes = 128 / BITS;  // codes in one 16-byte piece
@@ -311,11 +312,12 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
   // which of the four result registers holds this lane's diagonal element
   const int diag = (lane & 15) - 4 * (lane >> 4);
 
-  // rows are dealt to wavefronts in contiguous, balanced runs
-  const int64_t n_waves = (int64_t)gridDim.x * (blockDim.x / kWave);
-  const int64_t wave_id = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  const int64_t row_begin = wave_id * N / n_waves;
-  const int64_t row_end = (wave_id + 1) * N / n_waves;
+  // rows are dealt to wavefronts in contiguous, balanced runs: rows_per_wave
+  // each, one more for the first extra_rows wavefronts (the split is computed
+  // on the host: an integer division here would delay the first loads)
+  const int wave_id = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  const int64_t row_begin = (int64_t)wave_id * rows_per_wave + min(wave_id, extra_rows);
+  const int64_t row_end = row_begin + rows_per_wave + (wave_id < extra_rows ? 1 : 0);
   if (row_begin >= row_end) return;
   const char* wbytes = reinterpret_cast<const char*>(wq);
 
@@ -422,9 +424,11 @@ int launch_rows_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, 
   int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
   const int64_t max_blocks = (N + 3) / 4;  // at least one row per wavefront
   if (blocks > max_blocks) blocks = max_blocks;
+  const int64_t n_waves = blocks * 4;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
-                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, gs_shift);
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, gs_shift, (int)(N / n_waves),
+                     (int)(N % n_waves));
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 

@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
                                                                       uint16_t* __restrict__ biases,
                                                                       int64_t n_groups) {
   constexpr int kChunks = GS / 8;                 // 16-byte pieces per group
-  constexpr int kWordsPerChunk = BITS / 4;        // packed words produced per piece
+  constexpr int kWords = GS * BITS / 32;          // packed words per group
   constexpr float n_bins = (float)((1 << BITS) - 1);
   __shared__ uint4 stage_all[4][kWave * kChunks];
   const int lane = threadIdx.x & (kWave - 1);
@@ -264,16 +264,23 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
     const uint32_t er = exponent_field(range), ee = exponent_field(edge);
     const bool tame = (er - 64u) <= 126u && (ee - 64u) <= 126u && ee <= er + 40u;  // see quantize_kernel
     float scale, bias = 0.0f;
-    uint32_t words[kChunks * kWordsPerChunk];
-    auto pack = [&](int i, const uint32_t (&code)[8]) {
-      if constexpr (BITS == 4) {
-        uint32_t word = 0;
+    // The group's codes form one little-endian bit stream, code i at bit
+    // i*BITS: for 4 and 8 bits that is "element i of a word at bit i*BITS", for
+    // 3, 5 and 6 bits it is MLX's 3- and 5-byte packs laid end to end.  The
+    // loops are fully unrolled, so every shift and index below is a constant.
+    uint32_t words[kWords];
+    uint64_t stream = 0;
+    int stream_bits = 0, n_words = 0;
+    auto pack = [&](int, const uint32_t (&code)[8]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) word |= code[e] << (4 * e);
-        words[i] = word;
-      } else {
-        words[2 * i] = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
-        words[2 * i + 1] = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+      for (int e = 0; e < 8; ++e) {
+        stream |= (uint64_t)code[e] << stream_bits;
+        stream_bits += BITS;
+        if (stream_bits >= 32) {
+          words[n_words++] = (uint32_t)stream;
+          stream >>= 32;
+          stream_bits -= 32;
+        }
       }
     };
     if (tame) {
@@ -320,10 +327,18 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
     }
     const int64_t g = g0 + lane;
     if (g < n_groups) {
-      uint4* out = reinterpret_cast<uint4*>(wq + g * (kChunks * kWordsPerChunk));
+      uint32_t* out = wq + g * kWords;  // 4 * kWords bytes per group: the widest store that stays aligned
+      if constexpr (kWords % 4 == 0) {
 #pragma unroll
-      for (int k = 0; k < kChunks * kWordsPerChunk / 4; ++k)
-        out[k] = make_uint4(words[4 * k], words[4 * k + 1], words[4 * k + 2], words[4 * k + 3]);
+        for (int k = 0; k < kWords / 4; ++k)
+          reinterpret_cast<uint4*>(out)[k] = make_uint4(words[4 * k], words[4 * k + 1], words[4 * k + 2], words[4 * k + 3]);
+      } else if constexpr (kWords % 2 == 0) {
+#pragma unroll
+        for (int k = 0; k < kWords / 2; ++k) reinterpret_cast<uint2*>(out)[k] = make_uint2(words[2 * k], words[2 * k + 1]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) out[k] = words[k];
+      }
       scales[g] = T::from_f32(scale);
       biases[g] = T::from_f32(bias);
     }
@@ -424,6 +439,60 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(const uint32_t* __
   }
 }
 
+// 3-, 5- and 6-bit codes: a thread takes 32 consecutive elements, which are
+// BITS whole words of the row's bit stream, and unpacks them with constant
+// shifts.  idx == nullptr: plain dequantize over n_units units; otherwise unit
+// u of looked-up row blockIdx.y comes from row idx[blockIdx.y] (see
+// dequantize_rows_kernel).
+template <typename TS, typename TO, int GS, int BITS>
+__global__ __launch_bounds__(256) void dequantize_stream_kernel(const uint32_t* __restrict__ wq,
+                                                                const typename TS::storage* __restrict__ scales,
+                                                                const typename TS::storage* __restrict__ biases,
+                                                                const int64_t* __restrict__ idx, int64_t n_rows,
+                                                                int64_t units_per_row, int64_t n_units,
+                                                                typename TO::storage* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; u < n_units; u += stride) {
+    int64_t src = u, dst = u;
+    if (idx) {
+      int64_t row = idx[blockIdx.y];
+      if (row < 0) row += n_rows;
+      row = row < 0 ? 0 : (row >= n_rows ? n_rows - 1 : row);
+      src = row * units_per_row + u;
+      dst = (int64_t)blockIdx.y * units_per_row + u;
+    }
+    const float s = TS::to_f32(scales[src * 32 / GS]);
+    const float b = TS::to_f32(biases[src * 32 / GS]);
+    uint32_t w[BITS + 1];
+#pragma unroll
+    for (int i = 0; i < BITS; ++i) w[i] = wq[src * BITS + i];
+    w[BITS] = 0;
+    float r[32];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+      const int bit = e * BITS, word = bit / 32, sh = bit % 32;
+      uint32_t code = w[word] >> sh;
+      if (sh + BITS > 32) code |= w[word + 1] << (32 - sh);
+      r[e] = __builtin_fmaf((float)(code & ((1u << BITS) - 1u)), s, b);
+    }
+    if constexpr (sizeof(typename TO::storage) == 2) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        uint4 o;
+        o.x = TO::pack2(r[8 * k], r[8 * k + 1]);
+        o.y = TO::pack2(r[8 * k + 2], r[8 * k + 3]);
+        o.z = TO::pack2(r[8 * k + 4], r[8 * k + 5]);
+        o.w = TO::pack2(r[8 * k + 6], r[8 * k + 7]);
+        reinterpret_cast<uint4*>(out)[4 * dst + k] = o;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        reinterpret_cast<float4*>(out)[8 * dst + k] = make_float4(r[4 * k], r[4 * k + 1], r[4 * k + 2], r[4 * k + 3]);
+    }
+  }
+}
+
 int grid_for(int64_t n_chunks, int per_thread) {
   const int64_t blocks = (n_chunks + 256LL * per_thread - 1) / (256LL * per_thread);
   const int64_t cap = 256 * 8;  // 8 workgroups per CU keeps ~128 KiB of loads in flight per CU
@@ -439,14 +508,18 @@ int quantize_bits(const void* w, int64_t n_chunks, int bits, uint32_t* wq, void*
     const int64_t blocks = (n_groups + 4 * kWave - 1) / (4 * kWave);  // four wavefronts of 64 groups each
     const int64_t cap = 256 * 4;  // resident at once on 256 CUs; wavefronts loop over the rest
     const int grid = (int)(blocks < cap ? blocks : cap);
-    if (bits == 4) {
-      hipLaunchKernelGGL((quantize_group_per_lane_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq,
-                         (S*)scales, (S*)biases, n_groups);
-    } else {
-      hipLaunchKernelGGL((quantize_group_per_lane_kernel<T, GS, 8>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq,
-                         (S*)scales, (S*)biases, n_groups);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales, (S*)biases, n_groups);
+    };
+    switch (bits) {
+      case 3: launch(quantize_group_per_lane_kernel<T, GS, 3>); break;
+      case 4: launch(quantize_group_per_lane_kernel<T, GS, 4>); break;
+      case 5: launch(quantize_group_per_lane_kernel<T, GS, 5>); break;
+      case 6: launch(quantize_group_per_lane_kernel<T, GS, 6>); break;
+      default: launch(quantize_group_per_lane_kernel<T, GS, 8>); break;
     }
   } else {
+    if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;  // float32 input: 4 and 8 bits only
     const int grid = grid_for(n_chunks, kUnroll);
     if (bits == 4) {
       hipLaunchKernelGGL((quantize_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
@@ -475,7 +548,17 @@ int dequantize_bits(const uint32_t* wq, const void* scales, const void* biases, 
   using SS = typename TS::storage;
   using SO = typename TO::storage;
   const int grid = grid_for(n_chunks, 1);
-  if (bits == 4) {
+  if (bits == 3 || bits == 5 || bits == 6) {
+    const int64_t n_units = n_chunks / 4;  // 32 elements each
+    const int g = grid_for(n_units, 1);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(g), dim3(256), 0, stream, wq, (const SS*)scales, (const SS*)biases,
+                         (const int64_t*)nullptr, (int64_t)0, (int64_t)0, n_units, (SO*)out);
+    };
+    if (bits == 3) launch(dequantize_stream_kernel<TS, TO, GS, 3>);
+    if (bits == 5) launch(dequantize_stream_kernel<TS, TO, GS, 5>);
+    if (bits == 6) launch(dequantize_stream_kernel<TS, TO, GS, 6>);
+  } else if (bits == 4) {
     hipLaunchKernelGGL((dequantize_kernel<TS, TO, GS, 4>), dim3(grid), dim3(256), 0, stream, wq, (const SS*)scales,
                        (const SS*)biases, (SO*)out, n_chunks);
   } else {
@@ -500,7 +583,18 @@ int dequantize_rows_bits(const uint32_t* wq, const void* scales, const void* bia
                          int64_t n_rows, int chunks_per_row, int bits, void* out, hipStream_t stream) {
   using SS = typename TS::storage;
   using SO = typename TO::storage;
-  if (bits == 4) {
+  if (bits == 3 || bits == 5 || bits == 6) {
+    if (n_idx > 65535) return MFQ_EUNSUPPORTED;  // looked-up rows ride on gridDim.y
+    const int64_t upr = chunks_per_row / 4;
+    const dim3 g((unsigned)((upr + 255) / 256), (unsigned)n_idx);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, g, dim3(256), 0, stream, wq, (const SS*)scales, (const SS*)biases, idx, n_rows, upr,
+                         upr, (SO*)out);
+    };
+    if (bits == 3) launch(dequantize_stream_kernel<TS, TO, GS, 3>);
+    if (bits == 5) launch(dequantize_stream_kernel<TS, TO, GS, 5>);
+    if (bits == 6) launch(dequantize_stream_kernel<TS, TO, GS, 6>);
+  } else if (bits == 4) {
     hipLaunchKernelGGL((dequantize_rows_kernel<TS, TO, GS, 4>), dim3((unsigned)n_idx), dim3(256), 0, stream, wq,
                        (const SS*)scales, (const SS*)biases, idx, n_rows, chunks_per_row, (SO*)out);
   } else {

@@ -99,7 +99,7 @@ static inline void store_from_f32(void* p, int dtype, size_t i, float v) {
 static int check_args(int dtype, int group_size, int bits) {
   if (dtype < 0 || dtype > 2) return -1;
   if (group_size != 32 && group_size != 64 && group_size != 128) return -2;
-  if (bits != 2 && bits != 4 && bits != 8) return -3; /* power-of-two widths */
+  if (bits != 2 && bits != 3 && bits != 4 && bits != 5 && bits != 6 && bits != 8) return -3;
   return 0;
 }
 
@@ -115,9 +115,15 @@ int mlxo_quantize(const void* w, int dtype, size_t n_elem, int group_size,
   if (rc) return rc;
   if (n_elem % (size_t)group_size) return -4;
   const float n_bins = (float)((1 << bits) - 1);
-  const int el_per_int = 32 / bits;
-  const int int_per_group = group_size / el_per_int;
+  /* MLX packs el_per_pack codes into bytes_per_pack bytes, lowest code in the
+   * lowest bits: 32/bits codes per 4 bytes for 2, 4, 8 bits; 8 codes per 3
+   * bytes (3 bits), 8 per 5 (5 bits), 4 per 3 (6 bits).                      */
+  const int pow2 = (bits & (bits - 1)) == 0;
+  const int el_per_pack = pow2 ? 32 / bits : (bits == 6 ? 4 : 8);
+  const int bytes_per_pack = pow2 ? 4 : (bits == 5 ? 5 : 3);
+  const int packs_per_group = group_size / el_per_pack;
   const size_t n_groups = n_elem / (size_t)group_size;
+  uint8_t* out_bytes = (uint8_t*)out;
 
   /* groups are independent; the thread split changes nothing in the results */
 #pragma omp parallel for schedule(static) if (n_groups > 4096)
@@ -141,17 +147,17 @@ int mlxo_quantize(const void* w, int dtype, size_t n_elem, int group_size,
       scale = edge / q0;
       bias = edge;
     }
-    uint32_t* o = out + g * (size_t)int_per_group;
-    for (int j = 0; j < int_per_group; ++j) {
-      uint32_t word = 0;
-      for (int k = 0; k < el_per_int; ++k) {
-        float e = load_as_f32(w, dtype, w_idx + (size_t)j * el_per_int + k);
+    uint8_t* o = out_bytes + g * (size_t)packs_per_group * bytes_per_pack;
+    for (int j = 0; j < packs_per_group; ++j) {
+      uint64_t pack = 0;
+      for (int k = 0; k < el_per_pack; ++k) {
+        float e = load_as_f32(w, dtype, w_idx + (size_t)j * el_per_pack + k);
         float q = MLXO_ROUND(MLXO_CODE(e, bias, scale));
         q = (q < 0.0f) ? 0.0f : q;     /* std::max(q, 0) */
         q = (n_bins < q) ? n_bins : q; /* std::min(q, n_bins) */
-        word |= (uint32_t)q << MLXO_SHIFT(k, bits);
+        pack |= (uint64_t)q << MLXO_SHIFT(k, bits);
       }
-      o[j] = word;
+      for (int b = 0; b < bytes_per_pack; ++b) o[j * bytes_per_pack + b] = (uint8_t)(pack >> (8 * b));
     }
     store_from_f32(scales, dtype, g, scale);
     store_from_f32(biases, dtype, g, bias);
@@ -159,10 +165,14 @@ int mlxo_quantize(const void* w, int dtype, size_t n_elem, int group_size,
   return 0;
 }
 
+/* code idx of a buffer: bits [idx*bits, (idx+1)*bits) of its little-endian
+ * bit stream (which is what both packing schemes above produce)            */
 static inline uint32_t code_at(const uint32_t* wq, size_t idx, int bits) {
-  const int el_per_int = 32 / bits;
-  uint32_t word = wq[idx / el_per_int];
-  return (word >> MLXO_SHIFT(idx % el_per_int, bits)) & ((1u << bits) - 1u);
+  const uint8_t* bytes = (const uint8_t*)wq;
+  const size_t bit = idx * (size_t)bits;
+  uint32_t window = bytes[bit >> 3];
+  if ((bit & 7) + (size_t)bits > 8) window |= (uint32_t)bytes[(bit >> 3) + 1] << 8;
+  return (window >> (bit & 7)) & ((1u << bits) - 1u);
 }
 
 /*
@@ -231,6 +241,7 @@ int mlxo_qmm_t_f32acc(const void* x, int x_dtype, size_t M, size_t K,
                       int threads) {
   int rc = check_args(sb_dtype, group_size, bits);
   if (rc) return rc;
+  if (bits & (bits - 1)) return -3; /* word-wise loop: 2, 4, 8 bits only */
   if (K % (size_t)group_size) return -4;
   const int el_per_int = 32 / bits;
   const size_t words_per_row = K / el_per_int;
@@ -285,6 +296,7 @@ int mlxo_qmm_t_tacc(const void* x, size_t M, size_t K, const uint32_t* wq,
                     size_t N, int group_size, int bits, void* y) {
   int rc = check_args(dtype, group_size, bits);
   if (rc) return rc;
+  if (bits & (bits - 1)) return -3; /* word-wise loop: 2, 4, 8 bits only */
   if (dtype == MLXO_F32) return -1;
   const int el_per_int = 32 / bits;
   const size_t words_per_row = K / el_per_int;

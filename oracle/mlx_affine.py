@@ -75,7 +75,7 @@ def _from_f32(x: np.ndarray, dtype: int) -> np.ndarray:
 def _check(group_size: int, bits: int) -> None:
     if group_size not in (32, 64, 128):
         raise ValueError(f"group_size {group_size} not supported")
-    if bits not in (2, 4, 8):
+    if bits not in (2, 3, 4, 5, 6, 8):
         raise ValueError(f"bits {bits} not supported")
 
 
@@ -108,23 +108,36 @@ def quantize(w: np.ndarray, dtype: int = BF16, group_size: int = 64, bits: int =
         bias = np.where(nz, edge, np.float32(0)).astype(np.float32)
         codes = np.rint((f - bias[:, None]) / scale[:, None])
         codes = np.minimum(np.maximum(codes, np.float32(0)), n_bins).astype(np.uint32)
-    per = 32 // bits
-    codes = codes.reshape(-1, per)
-    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))[None, :]
-    words = np.bitwise_or.reduce(codes << shifts, axis=1).astype(np.uint32)
+    words = pack_bitstream(codes.reshape(-1, K), bits)
     wq = words.reshape(*lead, K * bits // 32)
     scales = _from_f32(scale, dtype).reshape(*lead, K // group_size)
     biases = _from_f32(bias, dtype).reshape(*lead, K // group_size)
     return wq, scales, biases
 
 
+def pack_bitstream(codes: np.ndarray, bits: int) -> np.ndarray:
+    """codes [R, K] -> uint32 [R, K*bits/32]: every row is one little-endian bit
+    stream in which code i occupies bits [i*bits, (i+1)*bits).  For 2, 4 and 8
+    bits that is MLX's "element i of a word at bit offset i*bits"; for 3, 5 and
+    6 bits it is MLX's byte packs (8 codes in 3 bytes, 8 in 5, 4 in 3), whose
+    boundaries fall on whole bytes of the same stream."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint32)
+    rows, K = codes.shape
+    bit = ((codes[:, :, None] >> np.arange(bits, dtype=np.uint32)) & np.uint32(1)).astype(np.uint8)
+    stream = np.packbits(bit.reshape(rows, K * bits), axis=1, bitorder="little")
+    return np.ascontiguousarray(stream).view(np.uint32).reshape(rows, K * bits // 32)
+
+
 def unpack_codes(wq: np.ndarray, bits: int) -> np.ndarray:
-    """uint32 [..., W] -> uint32 codes [..., W*32/bits], element i of a word at
-    bit offset i*bits."""
-    per = 32 // bits
-    shifts = np.arange(per, dtype=np.uint32) * np.uint32(bits)
-    codes = (wq[..., None] >> shifts) & np.uint32((1 << bits) - 1)
-    return codes.reshape(*wq.shape[:-1], wq.shape[-1] * per)
+    """uint32 [..., W] -> uint32 codes [..., W*32/bits], code i of a row at bit
+    offset i*bits of the row's little-endian bit stream."""
+    wq = np.ascontiguousarray(wq, dtype=np.uint32)
+    lead, W = wq.shape[:-1], wq.shape[-1]
+    stream = np.unpackbits(wq.reshape(-1, W).view(np.uint8), axis=1, bitorder="little")
+    n = W * 32 // bits
+    bit = stream[:, :n * bits].reshape(-1, n, bits).astype(np.uint32)
+    codes = (bit << np.arange(bits, dtype=np.uint32)).sum(axis=2, dtype=np.uint32)
+    return codes.reshape(*lead, n)
 
 
 def dequantize_exact(wq, scales, biases, dtype: int = BF16, group_size: int = 64, bits: int = 4) -> np.ndarray:
@@ -218,8 +231,8 @@ def c_dequantize(wq, scales, biases, dtype: int = BF16, group_size: int = 64, bi
     wq = np.ascontiguousarray(wq, dtype=np.uint32)
     scales = np.ascontiguousarray(scales)
     biases = np.ascontiguousarray(biases)
-    n = wq.size * (32 // bits)
-    out = np.empty((*wq.shape[:-1], wq.shape[-1] * (32 // bits)), dtype=_storage(out_dtype))
+    n = wq.size * 32 // bits
+    out = np.empty((*wq.shape[:-1], wq.shape[-1] * 32 // bits), dtype=_storage(out_dtype))
     rc = clib().mlxo_dequantize(_ptr(wq), _ptr(scales), _ptr(biases), dtype, n, group_size, bits, _ptr(out), out_dtype)
     if rc:
         raise ValueError(f"mlxo_dequantize failed with {rc}")
@@ -230,8 +243,8 @@ def c_dequantize_f64(wq, scales, biases, dtype: int = BF16, group_size: int = 64
     wq = np.ascontiguousarray(wq, dtype=np.uint32)
     scales = np.ascontiguousarray(scales)
     biases = np.ascontiguousarray(biases)
-    n = wq.size * (32 // bits)
-    out = np.empty((*wq.shape[:-1], wq.shape[-1] * (32 // bits)), dtype=np.float64)
+    n = wq.size * 32 // bits
+    out = np.empty((*wq.shape[:-1], wq.shape[-1] * 32 // bits), dtype=np.float64)
     rc = clib().mlxo_dequantize_f64(_ptr(wq), _ptr(scales), _ptr(biases), dtype, n, group_size, bits, _ptr(out))
     if rc:
         raise ValueError(f"mlxo_dequantize_f64 failed with {rc}")

@@ -60,20 +60,20 @@ def test_argument_validation_needs_no_device():
     base = (ctypes.addressof(buf) + 15) & ~15
     q = lib.mfq_quantize_affine
     assert q(base, _lib.BF16, 4, 64, 48, 4, base, base, base, None) == E["group"]
-    assert q(base, _lib.BF16, 4, 64, 64, 5, base, base, base, None) == E["bits"]
+    assert q(base, _lib.BF16, 4, 64, 64, 7, base, base, base, None) == E["bits"]
     assert q(base, 7, 4, 64, 64, 4, base, base, base, None) == E["dtype"]
     assert q(base, _lib.BF16, 4, 96, 64, 4, base, base, base, None) == E["shape"]
     assert q(base, _lib.BF16, 0, 64, 64, 4, base, base, base, None) == E["shape"]
     assert q(None, _lib.BF16, 4, 64, 64, 4, base, base, base, None) == E["null"]
     assert q(base + 2, _lib.BF16, 4, 64, 64, 4, base, base, base, None) == E["align"]
     d = lib.mfq_dequantize_affine
-    assert d(base, base, base, _lib.BF16, 4, 64, 64, 3, base, _lib.BF16, None) == E["bits"]
+    assert d(base, base, base, _lib.BF16, 4, 64, 64, 2, base, _lib.BF16, None) == E["bits"]
     assert d(base, base, None, _lib.BF16, 4, 64, 64, 4, base, _lib.BF16, None) == E["null"]
     g = lib.mfq_dequantize_rows
     assert g(base, base, base, _lib.BF16, None, 2, 10, 128, 64, 4, base, _lib.BF16, None) == E["null"]
     assert g(base, base, base, _lib.BF16, base, 0, 10, 128, 64, 4, base, _lib.BF16, None) == E["shape"]
     assert g(base, base, base, _lib.BF16, base, 2, 10, 100, 64, 4, base, _lib.BF16, None) == E["shape"]
-    assert g(base, base, base, _lib.BF16, base, 2, 10, 128, 64, 6, base, _lib.BF16, None) == E["bits"]
+    assert g(base, base, base, _lib.BF16, base, 2, 10, 128, 64, 7, base, _lib.BF16, None) == E["bits"]
     m = lib.mfq_qmm_t
     args = dict(x=base, xd=_lib.BF16, M=4, K=128, wq=base, s=base, b=base, sd=_lib.BF16, bias=None, N=8, gs=64,
                 bits=4, y=base, yd=_lib.BF16, stream=None)
@@ -92,6 +92,7 @@ def test_argument_validation_needs_no_device():
     assert call(wq=None) == E["null"]
     assert call(x=base + 4) == E["align"]
     assert call(gs=16) == E["group"]
+    assert call(bits=5) == -8                        # 3, 5, 6 bits: no fused matmul kernel
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

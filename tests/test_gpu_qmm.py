@@ -146,6 +146,29 @@ def test_qmm_k_not_multiple_of_64(oracle, bits):
     _assert_close(_run(o, *args, bits, 32), _ref(o, *args, bits, 32))
 
 
+@pytest.mark.parametrize("bits", [3, 5, 6])
+@pytest.mark.parametrize("M", [1, 300])
+def test_odd_bit_widths_matmul(oracle, bits, M):
+    """3, 5, 6 bits: dequantize kernel + library GEMM, to the same tolerance,
+    through the functional API and through a QuantizedLinear."""
+    import mflux_amd
+    from gpu_util import to_dev
+    from mflux_amd import nn as qnn
+
+    o = oracle
+    args = _case(o, 13, M, 512, 192, bits)
+    ref = _ref(o, *args, bits)
+    _assert_close(_run(o, *args, bits), ref)
+    x, wq, s, b, bias = args
+    lin = qnn.Linear(512, 192, bias=True, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(to_dev(o.f32_to_bf16_bits(seeded(13, 1, (192, 512), 0.02)), o.BF16))
+        lin.bias.copy_(to_dev(bias, o.BF16))
+    q = lin.to_quantized(bits=bits)
+    assert q.bits == bits and tuple(q.weight.shape) == (192, 512 * bits // 32)
+    _assert_close(q(to_dev(x, o.BF16)), ref)
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 32), (8, 32), (4, 128), (8, 128)])
 def test_qmm_group_sizes(oracle, bits, gs):
     o = oracle

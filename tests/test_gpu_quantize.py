@@ -182,3 +182,55 @@ def test_quantized_embedding_module(oracle):
     ref = o.quantized_matmul_f64(x.double().cpu().numpy(), wq, s, b, o.BF16, 64, 8)
     err = np.abs(y.double().cpu().numpy() - ref).max(axis=1) / np.abs(ref).max(axis=1)
     assert tuple(y.shape) == (3, 500) and err.max() <= 1e-2
+
+
+@pytest.mark.parametrize("bits", [3, 5, 6])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_odd_bit_widths_quantize_and_dequantize_bit_exact(oracle, bits, gs, dtype_name):
+    """3-, 5- and 6-bit packing (MLX's byte packs): packed words, scales and
+    biases equal the oracle's; dequantize and the row lookup equal the
+    single-rounded fma of the oracle's codes."""
+    import mflux_amd
+    from gpu_util import TORCH_DT, raw, to_dev, u32_to_dev
+
+    o = oracle
+    dtype = {"bf16": o.BF16, "f16": o.F16}[dtype_name]
+    rows, K = 80, 1024
+    rnd = seeded(9, bits * 1000 + gs + 7, (rows, K), 0.02)
+    adv = _adversarial_groups(o, rows * K // gs, gs, seed=bits + gs + 1).reshape(rows, K)
+    for name, f32 in (("random", rnd), ("adversarial", adv)):
+        w = _storage(o, f32, dtype)
+        exp = o.c_quantize(w, dtype, gs, bits)
+        got = mflux_amd.quantize(to_dev(w, dtype), group_size=gs, bits=bits)
+        for what, e, g in zip(("wq", "scales", "biases"), exp, got):
+            assert tuple(g.shape) == e.shape, (name, what)
+            bad = np.flatnonzero(raw(g).reshape(-1) != e.reshape(-1))
+            assert bad.size == 0, f"{name}/{what}: {bad.size} mismatches, first at {bad[:4]}"
+    wq, s, b = exp
+    finite = np.isfinite(o.dequantize_exact(wq, s, b, dtype, gs, bits)).all(axis=1)
+    with np.errstate(all="ignore"):
+        fma32 = o.dequantize_exact(wq, s, b, dtype, gs, bits).astype(np.float32)
+    d32 = mflux_amd.dequantize(u32_to_dev(wq), to_dev(s, dtype), to_dev(b, dtype), group_size=gs, bits=bits,
+                               dtype=torch.float32)
+    assert np.array_equal(raw(d32)[finite], fma32[finite])
+    d16 = mflux_amd.dequantize(u32_to_dev(wq), to_dev(s, dtype), to_dev(b, dtype), group_size=gs, bits=bits)
+    assert d16.dtype == TORCH_DT[dtype] and torch.equal(d16[torch.from_numpy(finite).cuda()],
+                                                         d32.to(TORCH_DT[dtype])[torch.from_numpy(finite).cuda()])
+    idx = torch.tensor([[3, -1], [0, 500]], device="cuda")
+    looked = mflux_amd.dequantize_rows(u32_to_dev(wq), to_dev(s, dtype), to_dev(b, dtype), idx, group_size=gs,
+                                       bits=bits, dtype=torch.float32)
+    assert torch.equal(looked, d32[torch.tensor([[3, rows - 1], [0, rows - 1]], device="cuda")])
+
+
+def test_odd_bit_widths_full_size_weight(oracle):
+    """The 5-bit pack over a full FLUX attention weight."""
+    import mflux_amd
+    from gpu_util import raw, to_dev
+
+    o = oracle
+    w = o.f32_to_bf16_bits(seeded(3, 55, (3072, 3072), 0.02))
+    exp = o.c_quantize(w, o.BF16, 64, 5)
+    got = mflux_amd.quantize(to_dev(w, o.BF16), group_size=64, bits=5)
+    for e, g in zip(exp, got):
+        assert np.array_equal(raw(g), e)

@@ -27,6 +27,72 @@ def test_known_answers(oracle, impl, case):
     assert hex(int(b.reshape(-1)[0])) == hex(bias_bits)
 
 
+@pytest.mark.parametrize("impl", ["c", "numpy"])
+def test_known_answers_3_5_6_bits(oracle, impl):
+    """Byte packs of the odd widths, from closed forms worked out by hand
+    (tests/golden/README.md): a ramp that quantizes to codes 0, 1, 2, ... in
+    order, so pack j is a known integer written little-end first."""
+    o = oracle
+    fn = o.c_quantize if impl == "c" else o.quantize
+    # 3 bits: values (i-4)/8, codes 0..7 eight times; each 3-byte pack is 0xFAC688
+    vals = np.tile((np.arange(8, dtype=np.float32) - 4) / np.float32(8), 8)
+    wq, s, b = fn(o.f32_to_bf16_bits(vals).reshape(1, 64), o.BF16, 64, 3)
+    assert wq.shape == (1, 6) and s[0, 0] == 0x3E00 and b[0, 0] == 0xBF00
+    assert wq.view(np.uint8).reshape(-1).tolist() == [0x88, 0xC6, 0xFA] * 8
+    assert [hex(v) for v in wq.reshape(-1)[:3]] == ["0x88fac688", "0xc688fac6", "0xfac688fa"]
+    # 6 bits: values (i-32)/64, codes 0..63; pack j (4 codes, 3 bytes) = 0x0C2040 + j*0x104104
+    vals = (np.arange(64, dtype=np.float32) - 32) / np.float32(64)
+    wq, s, b = fn(o.f32_to_bf16_bits(vals).reshape(1, 64), o.BF16, 64, 6)
+    assert wq.shape == (1, 12) and s[0, 0] == 0x3C80 and b[0, 0] == 0xBF00
+    expect = []
+    for j in range(16):
+        v = 0x0C2040 + j * 0x104104
+        expect += [v & 0xFF, (v >> 8) & 0xFF, (v >> 16) & 0xFF]
+    assert wq.view(np.uint8).reshape(-1).tolist() == expect
+    # 5 bits: values (i-16)/32, codes 0..31 twice; pack j (8 codes, 5 bytes) = P0 + (j%4)*8*R,
+    # P0 = sum k*32^k (k<8), R = (32^8-1)/31
+    vals = np.tile((np.arange(32, dtype=np.float32) - 16) / np.float32(32), 2)
+    wq, s, b = fn(o.f32_to_bf16_bits(vals).reshape(1, 64), o.BF16, 64, 5)
+    assert wq.shape == (1, 10) and s[0, 0] == 0x3D00 and b[0, 0] == 0xBF00
+    p0, r = sum(k * 32 ** k for k in range(8)), (32 ** 8 - 1) // 31
+    assert (p0, r) == (0x398A418820, 0x842108421)
+    expect = []
+    for j in range(8):
+        v = p0 + (j % 4) * 8 * r
+        expect += [(v >> (8 * i)) & 0xFF for i in range(5)]
+    assert wq.view(np.uint8).reshape(-1).tolist() == expect
+
+
+@pytest.mark.parametrize("bits", [3, 5, 6])
+def test_odd_widths_restatements_agree_and_round_trip(oracle, bits):
+    o = oracle
+    n_bins = (1 << bits) - 1
+    for gs in (32, 64, 128):
+        w = o.f32_to_bf16_bits(seeded(9, 70 + bits, (32, 512), 0.02))
+        c, n = o.c_quantize(w, o.BF16, gs, bits), o.quantize(w, o.BF16, gs, bits)
+        assert c[0].shape == (32, 512 * bits // 32)
+        for a, b in zip(c, n):
+            assert np.array_equal(a, b)
+        codes = o.unpack_codes(c[0], bits)
+        assert codes.shape == (32, 512) and codes.max() == n_bins
+        assert np.array_equal(pack_stream(codes, bits), c[0])
+        assert np.array_equal(o.c_dequantize_f64(*c, o.BF16, gs, bits), o.dequantize_exact(*c, o.BF16, gs, bits))
+        err = np.abs(o.dequantize_exact(*c, o.BF16, gs, bits) - o.bf16_bits_to_f32(w))
+        step = np.repeat(np.abs(o.bf16_bits_to_f32(c[1])), gs, axis=1)
+        assert (err <= step * (1.0 + n_bins * 2.0 ** -9) + 1e-12).all()
+
+
+def pack_stream(codes, bits):
+    """Independent loop-based statement of the bit stream: python integers."""
+    out = []
+    for row in codes:
+        v = 0
+        for i, c in enumerate(row):
+            v |= int(c) << (i * bits)
+        out.append([(v >> (32 * j)) & 0xFFFFFFFF for j in range(len(row) * bits // 32)])
+    return np.array(out, dtype=np.uint32)
+
+
 def test_known_answers_as_float32_and_float16(oracle):
     """The same groups are exact in float16/float32, and the answers do not
     depend on the storage type beyond the final cast of scale and bias."""
@@ -236,7 +302,7 @@ def test_argument_errors(oracle):
     with pytest.raises(ValueError):
         o.quantize(np.zeros((4, 128), dtype=np.uint16), o.BF16, 48, 4)
     with pytest.raises(ValueError):
-        o.c_quantize(np.zeros((4, 128), dtype=np.uint16), o.BF16, 64, 5)
+        o.c_quantize(np.zeros((4, 128), dtype=np.uint16), o.BF16, 64, 7)
 
 
 # ---------------------------------------------------------------------------
