@@ -127,6 +127,28 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
               int sb_dtype, const void* bias, int64_t N, int group_size,
               int bits, void* y, int y_dtype, void* stream);
 
+/*
+ * mfq_qmm_t with an optional float32 workspace.  Has no counterpart in the
+ * reference (MLX allocates inside its ops).  Shapes with far fewer 256 x 256
+ * output tiles than the GPU has compute units -- the text-stream linears of the
+ * double blocks, M = 256 or 512 tokens against N = 3072, e.g.
+ * src/mflux/models/qwen/model/qwen_transformer/qwen_transformer_block.py:36-37
+ * on the caption tokens -- leave most of the chip idle; with a workspace K is
+ * cut into ranges that run on different compute units, each range accumulates
+ * into its own float32 plane of the workspace, and a second kernel adds the
+ * planes, rounds and applies the bias (same two roundings as the fused
+ * epilogue).  mfq_qmm_t_workspace_bytes() returns the size this shape would
+ * use on the current device (0: K is not split, pass NULL).  A NULL or smaller
+ * workspace is not an error: the call then runs as mfq_qmm_t does.  The
+ * workspace must be 16-byte aligned; its contents before and after the call
+ * are undefined; calls sharing one workspace must be ordered on one stream.
+ */
+size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits);
+int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
+                 const void* scales, const void* biases, int sb_dtype, const void* bias, int64_t N,
+                 int group_size, int bits, void* y, int y_dtype, void* workspace,
+                 size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,6 +22,9 @@ SIGNATURES = {
     "mfq_dequantize_affine": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_dequantize_rows": (_INT, [_PTR, _PTR, _PTR, _INT, _PTR, _I64, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
+    "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,
+                            ctypes.c_size_t, _PTR]),
 }
 
 _lib = None

@@ -232,11 +232,18 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
         if bias is not None:
             y = y + bias.to(y.dtype)
         return y.reshape(*lead, N)
+    lib = _lib.load()
     with torch.cuda.device(x.device):
-        rc = _lib.load().mfq_qmm_t(
+        # few output tiles (text-stream shapes): K is split across compute units
+        # through a float32 scratch, taken from torch's caching allocator on the
+        # current stream (so its reuse is ordered after this call)
+        ws_bytes = lib.mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+        rc = lib.mfq_qmm_t_ws(
             x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
             _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
-            y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device),
+            y.data_ptr(), _DTYPE_CODE[out_dtype], ws.data_ptr() if ws is not None else None, ws_bytes,
+            _stream_ptr(x.device),
         )
-    _lib.check("mfq_qmm_t", rc)
+    _lib.check("mfq_qmm_t_ws", rc)
     return y.reshape(*lead, N)

@@ -69,9 +69,22 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
                                      out, out_dtype, (hipStream_t)stream);
 }
 
+size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits) {
+  if (check_common(group_size, bits) != MFQ_OK || (bits != 4 && bits != 8)) return 0;
+  if (M <= 16 || N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  return mfq::qmm_workspace_bytes(M, N, K, group_size);
+}
+
 int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
               const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
               int y_dtype, void* stream) {
+  return mfq_qmm_t_ws(x, x_dtype, M, K, wq, scales, biases, sb_dtype, bias, N, group_size, bits, y, y_dtype, nullptr, 0,
+                      stream);
+}
+
+int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                 const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
+                 int y_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
   if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;  // 3, 5, 6 bits: dequantize, then a plain GEMM
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
@@ -96,8 +109,8 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* 
     }
     return MFQ_OK;
   }
-  return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
-                         (hipStream_t)stream);
+  return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, workspace,
+                         workspace_bytes, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -125,8 +125,11 @@ int launch_dequantize_rows(const uint32_t* wq, const void* scales, const void* b
 int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream);
+// workspace: optional float32 scratch for the K-split of shapes with few output
+// tiles (qmm_workspace_bytes() says how much; without it K is not split)
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               hipStream_t stream);
+               void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 
 }  // namespace mfq

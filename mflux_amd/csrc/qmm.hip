@@ -127,30 +127,35 @@ template <typename T, int GS, int BITS, bool kFast>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
-    int N, int K, int tiles_m, int tiles_n) {
+    int N, int K, int tiles_m, int tiles_n, int splits, int steps) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   using WR = WeightRegs<T, GS, BITS>;
   using SR = ScaleRegs<T, GS>;
 
   const int n_tiles = tiles_m * tiles_n;
+  const int n_items = n_tiles * splits;  // work items: (tile, k range); splits == 1 unless the launcher split K
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
   const int wn = wave * 64;
   const int r = lane & 31;
   const int h = lane >> 5;
-  const int steps = K / BK;
+  // `steps`: k steps of one work item (K / BK when K is not split)
 
-  // Persistent workgroups: workgroup b takes tiles b, b + grid, b + 2*grid, ...
+  // Persistent workgroups: workgroup b takes items b, b + grid, b + 2*grid, ...
+  // Item i is k range i / n_tiles of tile i % n_tiles: with K split, range s of
+  // every tile goes to float32 plane s of the workspace `y` points at, and a
+  // second kernel adds the planes up.
   // Workgroups are dealt round-robin to the 8 XCDs, so with a grid that is a
   // multiple of 8 a workgroup stays on XCD b%8 and that XCD's workgroups walk
   // a contiguous run of the tile sequence together.  Inside the run the tiles
   // are ordered in bands of kBandM tile-rows, row index fastest, so the ~32
   // tiles in flight on one XCD share kBandM x-tiles and 8 weight-tiles per k
   // step in that XCD's L2.
-  auto tile_origin = [&](int seq, int& m0, int& n0) {
-    int tile = seq;
+  auto tile_origin = [&](int seq, int& m0, int& n0, int& split) {
+    split = seq / n_tiles;
+    int tile = seq - split * n_tiles;
     const int per_xcd = n_tiles / 8;
     if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
     constexpr int kBandM = 4;
@@ -198,6 +203,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // x tile registers: set p receives the tile of a step with parity p, two
   // steps before it is used, and is published to LDS buffer p one step before.
   u32x4 xa[2][8];
+  char* y_item = static_cast<char*>(y);  // where the current item's results go
   WR wa, wb;            // packed weights of the current even / odd step
   SR sr;                // scales and biases of the period the prefetch cursor is in (kFast only)
   uint32_t bf[2][4];    // dequantised fragments of the next sub-step to run
@@ -348,19 +354,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // Fills the pipeline for the tile the prefetch offsets point at: x(0) into
   // LDS buffer 0, x(1) into register set 1, weights of steps 0 and 1, and the
   // fragments of sub-step 0.
-  auto prime = [&]() {
-    const int k1 = min(1, steps - 1) * BK;
+  auto prime = [&](int kb) {  // kb: first k of the item
+    const int k1 = kb + min(1, steps - 1) * BK;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xa[1][i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i]);
+    for (int i = 0; i < 8; ++i) xa[1][i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)kb * 2 + xoff[i]);
     if constexpr (kFast) {
-      sr.issue(scales, biases, soff, 0);
-      wa.issue_codes(wq, woff, 0);
+      sr.issue(scales, biases, soff, kb / GS);
+      wa.issue_codes(wq, woff, kb);
       wb.issue_codes(wq, woff, k1);
       sr.extract(wa, 0, h);
       sr.extract(wb, 1, h);
-      if constexpr (SR::kPeriod == 2) sr.issue(scales, biases, soff, 4);  // steps >= 4 here
+      if constexpr (SR::kPeriod == 2) sr.issue(scales, biases, soff, kb / GS + 4);  // steps >= 4 here
     } else {
-      wa.issue(wq, scales, biases, woff, soff, 0);
+      wa.issue(wq, scales, biases, woff, soff, kb);
       wb.issue(wq, scales, biases, woff, soff, k1);
     }
 #pragma unroll
@@ -407,7 +413,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           for (int c = 0; c < 4; ++c) v[c] = acc[ai][j][4 * eb + c];
           const int64_t o = (int64_t)row * N + col;
           if (y_is_f32) {
-            float* dst = reinterpret_cast<float*>(y) + o;
+            float* dst = reinterpret_cast<float*>(y_item) + o;
             if (bias) {
 #pragma unroll
               for (int c = 0; c < 4; ++c) v[c] += bv[c];
@@ -426,7 +432,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
               hv[c] = T::from_f32(v[c]);
               if (bias) hv[c] = T::from_f32(T::to_f32(hv[c]) + bv[c]);
             }
-            uint16_t* dst = reinterpret_cast<uint16_t*>(y) + o;
+            uint16_t* dst = reinterpret_cast<uint16_t*>(y_item) + o;
             if (n_vec_ok) {
               uint2 pk;
               pk.x = (uint32_t)hv[0] | ((uint32_t)hv[1] << 16);
@@ -461,7 +467,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int h = lane_e >> 5;
     const int lane = lane_e;
     char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
-    uint16_t* yout = reinterpret_cast<uint16_t*>(y);
+    uint16_t* yout = reinterpret_cast<uint16_t*>(y_item);
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
@@ -515,13 +521,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   };
 
   bool primed = false;
-  for (int seq = blockIdx.x; seq < n_tiles; seq += gridDim.x) {
-    int m0, n0;
-    tile_origin(seq, m0, n0);
+  for (int seq = blockIdx.x; seq < n_items; seq += gridDim.x) {
+    int m0, n0, split;
+    tile_origin(seq, m0, n0, split);
+    const int kb = split * steps * BK;            // first k of this item
+    constexpr int kGroupsPerStep2 = 2 * BK / GS;  // groups per step, times two (GS == 128: one)
+    const int gb = split * steps * kGroupsPerStep2 / 2;  // its first group
+    y_item = static_cast<char*>(y) + (size_t)split * M * N * 4;  // split > 0 only with float32 planes
     if (!primed) {
       set_scale_tile(n0);
       set_prefetch_tile(m0, n0);
-      prime();
+      prime(kb);
     }
     if constexpr (kFast) {
       // Pairs of steps (p, p+1), laid out period by period so that what each
@@ -533,7 +543,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       // the last pair.  Without a next tile those prefetches re-read pieces of
       // this tile and are never consumed.
       constexpr int kPer = SR::kPeriod;
-      constexpr int kGroupsPerStep2 = 2 * BK / GS;  // groups per step, times two (GS == 128: one)
       auto pair = [&](auto pos, int k_a, int g) __attribute__((always_inline)) {
         // pos: position of the pair's even step inside its period
         constexpr int kPos = decltype(pos)::value;
@@ -548,43 +557,45 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       // every pair of a period except its last two
       auto period_head = [&](int p) __attribute__((always_inline)) {
         if constexpr (kPer == 8) {
-          pair(std::integral_constant<int, 0>{}, (p + 2) * BK, 0);
-          pair(std::integral_constant<int, 2>{}, (p + 4) * BK, 0);
+          pair(std::integral_constant<int, 0>{}, kb + (p + 2) * BK, 0);
+          pair(std::integral_constant<int, 2>{}, kb + (p + 4) * BK, 0);
         }
       };
-      const bool has_next = seq + (int)gridDim.x < n_tiles;
+      const bool has_next = seq + (int)gridDim.x < n_items;
       for (int p = 0; p < steps - (kPer >= 4 ? kPer : 4); p += kPer) {
         period_head(p);
         if constexpr (kPer >= 4) {
-          pair(std::integral_constant<int, kPer - 4>{}, (p + kPer - 2) * BK, (p + kPer) * kGroupsPerStep2 / 2);
-          pair(std::integral_constant<int, kPer - 2>{}, (p + kPer) * BK, 0);
+          pair(std::integral_constant<int, kPer - 4>{}, kb + (p + kPer - 2) * BK, gb + (p + kPer) * kGroupsPerStep2 / 2);
+          pair(std::integral_constant<int, kPer - 2>{}, kb + (p + kPer) * BK, 0);
         } else {
-          pair(std::integral_constant<int, 0>{}, (p + 2) * BK, (p + 4) * kGroupsPerStep2 / 2);
+          pair(std::integral_constant<int, 0>{}, kb + (p + 2) * BK, gb + (p + 4) * kGroupsPerStep2 / 2);
         }
       }
       {
         const int p = steps - kPer;  // first step of the last period
-        int m1 = m0, n1 = n0;
-        if (has_next) tile_origin(seq + gridDim.x, m1, n1);
-        const int g_last = p * kGroupsPerStep2 / 2;  // this tile's last period, for prefetches nobody consumes
+        int m1 = m0, n1 = n0, split1 = split;
+        if (has_next) tile_origin(seq + gridDim.x, m1, n1, split1);
+        const int kb1 = split1 * steps * BK, gb1 = split1 * steps * kGroupsPerStep2 / 2;  // the next item's first k, group
+        const int g_last = gb + p * kGroupsPerStep2 / 2;  // this item's last period, for prefetches nobody consumes
+        const int k_last = kb + (steps - 2) * BK;
         if constexpr (kPer >= 4) {
           period_head(p);
           if (has_next) set_scale_tile(n1);
-          pair(std::integral_constant<int, kPer - 4>{}, (steps - 2) * BK, has_next ? 0 : g_last);
+          pair(std::integral_constant<int, kPer - 4>{}, k_last, has_next ? gb1 : g_last);
           if (has_next) set_prefetch_tile(m1, n1);
-          pair(std::integral_constant<int, kPer - 2>{}, has_next ? 0 : (steps - 2) * BK, 0);
+          pair(std::integral_constant<int, kPer - 2>{}, has_next ? kb1 : k_last, 0);
         } else {
           // the main loop stopped one period early: steps - 4 and steps - 2 remain
           if (has_next) set_scale_tile(n1);
-          pair(std::integral_constant<int, 0>{}, (steps - 2) * BK, has_next ? 0 : g_last);
+          pair(std::integral_constant<int, 0>{}, k_last, has_next ? gb1 : g_last);
           if (has_next) set_prefetch_tile(m1, n1);
-          pair(std::integral_constant<int, 0>{}, has_next ? 0 : (steps - 2) * BK, has_next ? 4 : g_last);
+          pair(std::integral_constant<int, 0>{}, has_next ? kb1 : k_last, has_next ? gb1 + 4 : g_last);
         }
       }
       primed = has_next;
     } else {
       int step = 0;
-      for (; step + 1 < steps; step += 2) {
+      for (; step + 1 < steps; step += 2) {  // never split: kb == 0
         do_step(even_step, keep, wa, wb, min(step + 2, steps - 1) * BK, 0, 0);
         do_step(odd_step, keep, wb, wa, min(step + 3, steps - 1) * BK, 0, 0);
       }
@@ -611,9 +622,83 @@ int compute_units() {
   return n;
 }
 
+// ---- K split across workgroups (few tiles, long K) -------------------------
+// With fewer than half as many 256 x 256 tiles as there are CUs, K is cut into
+// `splits` equal ranges of whole periods; range s of every tile is accumulated
+// into float32 plane s of a caller-provided workspace and the planes are added
+// up, rounded and biased by splitk_reduce_kernel.
+struct SplitPlan {
+  int splits;
+  int steps;  // k steps per range
+};
+
+// period: k steps per scale period of the group size.  The largest number of
+// equal ranges of whole periods (at least 4 steps each) that keeps one work
+// item per CU.
+inline SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int period, int cus) {
+  const int steps = (int)(K / BK);
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  SplitPlan plan{1, steps};
+  if (steps % period != 0 || steps < 4 || tiles * 2 > cus) return plan;
+  for (int s = 2; s <= steps / 4 && tiles * s <= cus; ++s)
+    if (steps % s == 0 && (steps / s) % period == 0) plan = SplitPlan{s, steps / s};
+  return plan;
+}
+
+inline int period_of(int gs) { return 4 * gs / BK; }
+
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ planes, int splits,
+                                                            int64_t plane_elems, const uint16_t* __restrict__ bias,
+                                                            int N, void* __restrict__ y, int y_is_f32) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  // four consecutive outputs per thread when rows are a multiple of four long
+  // (a quad then never straddles two rows), one otherwise
+  if ((N & 3) == 0) {
+    for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < plane_elems / 4; q += stride) {
+      float4 sum = reinterpret_cast<const float4*>(planes)[q];
+      for (int sp = 1; sp < splits; ++sp) {
+        const float4 v = reinterpret_cast<const float4*>(planes + sp * plane_elems)[q];
+        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+      }
+      const int col = (int)((q * 4) % N);
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[col + c]);
+      }
+      if (y_is_f32) {
+        reinterpret_cast<float4*>(y)[q] = make_float4(sum.x + bv[0], sum.y + bv[1], sum.z + bv[2], sum.w + bv[3]);
+      } else {  // round, then add the bias and round again, as the fused epilogue does
+        uint2 pk;
+        pk.x = T::pack2(sum.x, sum.y);
+        pk.y = T::pack2(sum.z, sum.w);
+        if (bias) {
+          pk.x = T::pack2(lo_f32<T>(pk.x) + bv[0], hi_f32<T>(pk.x) + bv[1]);
+          pk.y = T::pack2(lo_f32<T>(pk.y) + bv[2], hi_f32<T>(pk.y) + bv[3]);
+        }
+        reinterpret_cast<uint2*>(y)[q] = pk;
+      }
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < plane_elems; i += stride) {
+      float sum = planes[i];
+      for (int sp = 1; sp < splits; ++sp) sum += planes[sp * plane_elems + i];
+      const float bv = bias ? T::to_f32(bias[i % N]) : 0.f;
+      if (y_is_f32) {
+        reinterpret_cast<float*>(y)[i] = sum + bv;
+      } else {
+        uint16_t hv = T::from_f32(sum);
+        if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
+        reinterpret_cast<uint16_t*>(y)[i] = hv;
+      }
+    }
+  }
+}
+
 template <typename T, int GS, int BITS, bool kFast>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                  const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
+                  const void* bias, int64_t N, void* y, int y_dtype, SplitPlan plan, hipStream_t stream) {
   auto kernel = qmm_kernel<T, GS, BITS, kFast>;
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
   if (!configured) {
@@ -624,17 +709,18 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   }
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
-  const int n_tiles = tiles_m * tiles_n;
-  const int grid = n_tiles < compute_units() ? n_tiles : compute_units();  // one persistent workgroup per CU
+  const int n_items = tiles_m * tiles_n * plan.splits;
+  const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
-                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n);
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.splits, plan.steps);
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-               const void* bias, int64_t N, void* y, int y_dtype, hipStream_t stream) {
+               const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
+               hipStream_t stream) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   // period-wise scale loads: whole periods, at least two pairs of steps, and
@@ -642,35 +728,63 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   const int64_t steps = K / BK;
   constexpr int kPer = ScaleRegs<T, GS>::kPeriod;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
-  if (steps % kPer == 0 && steps >= 4 && aligned8)
-    return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
-  return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
+  if (!(steps % kPer == 0 && steps >= 4 && aligned8))
+    return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype,
+                                             SplitPlan{1, (int)steps}, stream);
+  const SplitPlan plan = plan_split(M, N, K, kPer, compute_units());
+  const size_t need = (size_t)plan.splits * M * N * sizeof(float);
+  if (plan.splits == 1 || !workspace || workspace_bytes < need || !aligned16(workspace))
+    return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype,
+                                            SplitPlan{1, (int)steps}, stream);
+  if (int rc = launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
+                                                stream))
+    return rc;
+  const int64_t plane = M * N;
+  const int64_t threads = (N & 3) == 0 ? plane / 4 : plane;
+  const int64_t blocks = (threads + 255) / 256;
+  const int cap = compute_units() * 8;
+  hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, stream,
+                     (const float*)workspace, plan.splits, plane, (const uint16_t*)bias, (int)N, y,
+                     (int)(y_dtype == MFQ_F32));
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                const void* bias, int64_t N, int bits, void* y, int y_dtype, hipStream_t stream) {
-  if (bits == 4) return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
-  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, stream);
+                const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
+                hipStream_t stream) {
+  if (bits == 4) return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
 }
 
 template <typename T>
 int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-              const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream) {
+              const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
+              hipStream_t stream) {
   switch (gs) {
-    case 32: return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, stream);
-    case 64: return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, stream);
-    default: return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, stream);
+    case 32: return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    case 64: return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    default: return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
   }
 }
 
 }  // namespace
 
+size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
+  if (K % BK) return 0;
+  const SplitPlan plan = plan_split(M, N, K, period_of(gs), compute_units());
+  return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+}
+
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               hipStream_t stream) {
-  if (dtype == MFQ_BF16) return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
-  if (dtype == MFQ_F16) return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+               void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (dtype == MFQ_BF16)
+    return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                           stream);
+  if (dtype == MFQ_F16)
+    return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                          stream);
   return MFQ_EDTYPE;
 }
 

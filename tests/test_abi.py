@@ -20,7 +20,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
-                 "mfq_qmm_t"):
+                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes"):
         assert must in names
 
 

@@ -137,6 +137,59 @@ def test_qmm_vs_f64(oracle, bits, M, K, N):
     _assert_close(_run(o, *args, bits), _ref(o, *args, bits))
 
 
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 32), (8, 128)])
+@pytest.mark.parametrize("M,K,N", [(512, 3072, 768), (256, 3072, 520), (300, 1024, 200), (40, 2048, 1024)])
+def test_qmm_split_k_shapes(oracle, bits, gs, M, K, N):
+    """Few output tiles and a long K: the launcher cuts K into ranges that run
+    on different compute units and a second kernel adds the float32 planes.
+    Same tolerance; bf16 and float32 output; with bias."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    assert _lib.load().mfq_qmm_t_workspace_bytes(M, K, N, gs, bits) >= 2 * M * N * 4, "this shape should be split"
+    args = _case(o, 14, M, K, N, bits, gs=gs)
+    ref = _ref(o, *args, bits, gs)
+    _assert_close(_run(o, *args, bits, gs), ref)
+    x, wq, s, b, bias = args
+    y32 = mflux_amd.quantized_matmul(to_dev(x, o.BF16).float(), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                     group_size=gs, bits=bits, bias=to_dev(bias, o.BF16))
+    assert y32.dtype == torch.float32
+    _assert_close(y32, ref, tol=5e-3)  # float32 output: only the weights' 16-bit rounding remains
+
+
+def test_qmm_split_k_matches_unsplit_through_c_abi(oracle):
+    """mfq_qmm_t (no workspace) and mfq_qmm_t_ws (split) on the same operands:
+    both within tolerance of the oracle and of each other; a too-small
+    workspace silently runs unsplit."""
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    M, K, N, bits = 512, 3072, 512, 4
+    x, wq, s, b, bias = _case(o, 15, M, K, N, bits)
+    ref = _ref(o, x, wq, s, b, bias, bits)
+    xd, wd, sd, bd, biasd = to_dev(x, o.BF16), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16), to_dev(bias, o.BF16)
+    need = lib.mfq_qmm_t_workspace_bytes(M, K, N, 64, bits)
+    assert need > 0
+    outs = []
+    for ws_bytes in (0, 16, need):
+        y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+        rc = lib.mfq_qmm_t_ws(xd.data_ptr(), _lib.BF16, M, K, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), _lib.BF16,
+                              biasd.data_ptr(), N, 64, bits, y.data_ptr(), _lib.BF16,
+                              ws.data_ptr() if ws_bytes else None, ws_bytes, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        _assert_close(y, ref)
+        outs.append(y)
+    assert torch.equal(outs[0], outs[1])                       # too small: same unsplit kernel
+    diff = (outs[0].float() - outs[2].float()).abs().max() / outs[0].float().abs().max()
+    assert float(diff) <= 1e-2
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 def test_qmm_k_not_multiple_of_64(oracle, bits):
     """Group size 32 allows K = 96: large M goes through the small-M kernel in
