@@ -93,6 +93,7 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
   if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
   if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
+  if (M > 16 && !mfq::aligned16(y)) return MFQ_EALIGN;  // the GEMM writes y in 16-byte pieces
   if (M <= 16)
     return mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                            (hipStream_t)stream);

@@ -508,6 +508,55 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
     }
   };
+  // float32 output with N a multiple of 4 (the planes of a K split, float32 y):
+  // the same transpose, 64 rows at a time; a staged row is 64 floats plus 16
+  // bytes of padding, which again spreads the 16-byte writes (32 rows at once)
+  // and reads (4 rows at once) over all banks.  Every global store instruction
+  // writes four complete 256-byte row segments.
+  auto store_tile_staged_f32 = [&](int m0, int n0) {
+    constexpr int kStride = 64 * 4 + 16;
+    static_assert(64 * kStride <= kStageBytes, "float32 staging must fit the region of the 16-bit one");
+    int lane_e = lane;  // opaque copy, see store_tile_staged
+    asm volatile("" : "+v"(lane_e));
+    const int r = lane_e & 31;
+    const int h = lane_e >> 5;
+    const int lane = lane_e;
+    char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
+    float* yout = reinterpret_cast<float*>(y_item);
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int eb = 0; eb < 4; ++eb) {
+          const int cl = 32 * j + 8 * eb + 4 * h;  // column inside the wavefront's 64
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (bias) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(n0 + wn + cl + c, N - 1)]);
+          }
+#pragma unroll
+          for (int a2 = 0; a2 < 2; ++a2) {
+            const int ai = 2 * pass + a2;
+            *reinterpret_cast<float4*>(stage + (32 * a2 + r) * kStride + cl * 4) =
+                make_float4(acc[ai][j][4 * eb] + bv[0], acc[ai][j][4 * eb + 1] + bv[1], acc[ai][j][4 * eb + 2] + bv[2],
+                            acc[ai][j][4 * eb + 3] + bv[3]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // read back row-wise: lane l takes 16 bytes (4 columns) of row 4*k + l/16
+      const int cg = n0 + wn + 4 * (lane & 15);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int rl = 4 * k + (lane >> 4);
+        const float4 v = *reinterpret_cast<const float4*>(stage + rl * kStride + 16 * (lane & 15));
+        const int row = m0 + 64 * pass + rl;
+        if (row < M && cg < N) *reinterpret_cast<float4*>(yout + (int64_t)row * N + cg) = v;
+        if (k & 1) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
   auto store_tile = [&](int m0, int n0) {
     if (!y_is_f32 && (N & 7) == 0) {
       if (bias) {
@@ -515,6 +564,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       } else {
         store_tile_staged(std::false_type{}, m0, n0);
       }
+    } else if (y_is_f32 && (N & 3) == 0) {
+      store_tile_staged_f32(m0, n0);
     } else {
       store_tile_direct(m0, n0);
     }
