@@ -172,9 +172,74 @@ def dequantize_rows(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
     return out.reshape(*indices.shape, K)
 
 
+def _matmul_untransposed(x, w, scales, biases, group_size, bits):
+    """``x @ dequantize(w)`` (``w`` packed ``[N, K*bits/32]``, ``x`` ``[..., N]``): the
+    product MLX computes for ``transpose=False``, which is what the gradient of a
+    quantized linear with respect to its input needs when a LoRA is trained on a
+    quantized base (src/mflux/models/common/training/lora/target_injector.py:30-33
+    wraps ``nn.QuantizedLinear`` in a trainable ``LoRALinear``).  Composed
+    from this library's dequantize kernel and the BLAS library's GEMM."""
+    _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
+    if w.ndim != 2:
+        raise NotImplementedError("[quantized_matmul] batched weights are not implemented in this build")
+    N = w.shape[0]
+    K = w.shape[1] * 32 // bits
+    if x.ndim < 1 or x.shape[-1] != N:
+        raise ValueError(
+            f"[quantized_matmul] Last dimension of first input with shape {tuple(x.shape)} does not match the "
+            f"expanded quantized matrix ({N}, {K}) computed from shape {tuple(w.shape)} with "
+            f"group_size={group_size}, bits={bits} and transpose=false"
+        )
+    _require_hip("quantized_matmul", x, "x")
+    out_dtype = torch.result_type(x, scales)
+    w_full = dequantize(w, scales, biases, group_size, bits)
+    if out_dtype == scales.dtype:
+        return torch.matmul(x.to(scales.dtype), w_full)
+    return torch.matmul(x.float(), w_full.float())
+
+
+class _QuantizedMatmulFunction(torch.autograd.Function):
+    """Makes the fused forward differentiable with respect to ``x`` (and to a
+    trainable ``bias``); the packed weight, scales and biases are constants."""
+
+    @staticmethod
+    def forward(ctx, x, w, scales, biases, bias, group_size, bits):
+        ctx.save_for_backward(w, scales, biases)
+        ctx.meta = (group_size, bits, x.dtype, bias is not None, bias.dtype if bias is not None else None)
+        return _quantized_matmul_forward(x, w, scales, biases, group_size, bits, bias)
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        w, scales, biases = ctx.saved_tensors
+        group_size, bits, x_dtype, has_bias, bias_dtype = ctx.meta
+        grad_x = grad_bias = None
+        if ctx.needs_input_grad[0]:
+            grad_x = _matmul_untransposed(grad_y, w, scales, biases, group_size, bits).to(x_dtype)
+        if has_bias and ctx.needs_input_grad[4]:
+            grad_bias = grad_y.reshape(-1, grad_y.shape[-1]).sum(dim=0).to(bias_dtype)
+        return grad_x, None, None, None, grad_bias, None, None
+
+
 def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
                      transpose: bool = True, group_size: int = 64, bits: int = 4, mode: str = "affine",
                      *, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ dequantize(w).T`` (``transpose=True``) or ``x @ dequantize(w)``; see
+    ``_quantized_matmul_forward``.  Differentiable with respect to ``x`` and
+    ``bias``."""
+    _check_mode("quantized_matmul", mode)
+    _check_group_bits("quantized_matmul", group_size, bits)
+    if not transpose:
+        if bias is not None:
+            raise ValueError("[quantized_matmul] bias is only fused for transpose=True")
+        return _matmul_untransposed(x, w, scales, biases, group_size, bits)
+    needs_grad = torch.is_grad_enabled() and (x.requires_grad or (bias is not None and bias.requires_grad))
+    if needs_grad:
+        return _QuantizedMatmulFunction.apply(x, w, scales, biases, bias, group_size, bits)
+    return _quantized_matmul_forward(x, w, scales, biases, group_size, bits, bias)
+
+
+def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                              group_size: int, bits: int, bias: torch.Tensor | None) -> torch.Tensor:
     """``x @ dequantize(w).T`` with float32 accumulation.
 
     ``x``: ``[..., K]``; ``w``: packed ``[N, K*bits/32]``.  The result has dtype
@@ -184,10 +249,6 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
     of ``mx.quantized_matmul``) fuses the add of ``QuantizedLinear`` into the
     kernel's epilogue with the same two roundings as a separate add.
     """
-    _check_mode("quantized_matmul", mode)
-    _check_group_bits("quantized_matmul", group_size, bits)
-    if not transpose:
-        raise NotImplementedError("[quantized_matmul] transpose=False (x @ w) is not implemented in this build")
     _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
     if w.ndim != 2:
         raise NotImplementedError("[quantized_matmul] batched weights are not implemented in this build")

@@ -350,3 +350,40 @@ def test_f16_path(oracle):
         y = mflux_amd.quantized_matmul(x, wq, s, b, bits=8)
         ref = o.quantized_matmul_f64(x.double().cpu().numpy(), raw(wq), raw(s), raw(b), o.F16, 64, 8)
         _assert_close(y, ref)
+
+
+@pytest.mark.parametrize("bits", [4, 8, 5])
+def test_transpose_false_and_input_gradient(oracle, bits):
+    """transpose=False is g @ dequantize(w); it is also the gradient of the
+    fused forward with respect to x, so a LoRA can be trained on a quantized
+    base.  Both against float64 on the exactly dequantized weight."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import nn as qnn
+
+    o = oracle
+    M, K, N = 40, 512, 192
+    x, wq, s, b, bias = _case(o, 16, M, K, N, bits)
+    wd, sd, bd = u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16)
+    w_exact = o.dequantize_exact(wq, s, b, o.BF16, 64, bits)                       # [N, K]
+    g = o.f32_to_bf16_bits(seeded(16, 5, (M, N), 1.0))
+    gx = mflux_amd.quantized_matmul(to_dev(g, o.BF16), wd, sd, bd, transpose=False, group_size=64, bits=bits)
+    assert tuple(gx.shape) == (M, K) and gx.dtype == torch.bfloat16
+    _assert_close(gx, o.bf16_bits_to_f32(g).astype(np.float64) @ w_exact)
+    with pytest.raises(ValueError, match="transpose=false"):
+        mflux_amd.quantized_matmul(to_dev(x, o.BF16), wd, sd, bd, transpose=False, group_size=64, bits=bits)
+
+    # autograd through a QuantizedLinear wrapped by a LoRA-style branch
+    q = qnn.QuantizedLinear(K, N, bias=True, bits=bits, device="cuda")
+    q.weight, q.scales, q.biases, q.bias = wd, sd, bd, to_dev(bias, o.BF16)
+    xt = to_dev(x, o.BF16).clone().requires_grad_(True)
+    a = (torch.randn(K, 4, device="cuda") * 0.05).to(torch.bfloat16).requires_grad_(True)
+    bl = (torch.randn(4, N, device="cuda") * 0.05).to(torch.bfloat16).requires_grad_(True)
+    y = q(xt) + (xt @ a) @ bl
+    y.backward(to_dev(g, o.BF16))
+    gf = o.bf16_bits_to_f32(g).astype(np.float64)
+    ref_gx = gf @ w_exact + (gf @ bl.detach().double().cpu().numpy().T) @ a.detach().double().cpu().numpy().T
+    _assert_close(xt.grad, ref_gx, tol=2e-2)   # two bf16-rounded terms added in bf16
+    assert a.grad is not None and bl.grad is not None and q.weight.grad is None
+    # and no autograd graph is built when nothing requires grad
+    assert not q(to_dev(x, o.BF16)).requires_grad
