@@ -2,7 +2,7 @@
 """Benchmark of the quantized-linear hot path on one MI355X.
 
 Step = one pass of the FLUX.1 single-stream block's quantized linears at
-1024x1024 (BASELINE config 3): x[4608,3072] @ W4[21504,3072]^T followed by
+1024x1024 (the configuration the headline metric is quoted on): x[4608,3072] @ W4[21504,3072]^T followed by
 x2[4608,15360] @ W4[3072,15360]^T, group size 64, bf16 activations, synthetic
 N(0,1) activations and N(0,0.02) weights quantized on the device by this
 library.  Prints ONE JSON line; `value` is TFLOP/s over the two GEMMs with all
@@ -11,7 +11,7 @@ operands resident in HBM.
 The same line carries
   roofline     - the W4A16 GEMM kernel against the dense bf16 MFMA peak, from
                  HIP-event timing of the launches in the timed region;
-  secondary    - the W8 dequant-GEMV (BASELINE config 2, M=1 and M=4) against
+  secondary    - the W8 dequant-GEMV (adaLN modulation shape, M=1 and M=4) against
                  the HBM peak, weights rotated through > 256 MB so the memory-
                  side cache cannot serve them, and the quantize/pack pass over
                  both block weights;

@@ -9,8 +9,8 @@
 // the 32x32x16 matrix-core instruction.
 //   - x goes HBM -> registers -> LDS (128-bit moves, one 64-wide k step ahead,
 //     two LDS buffers, one barrier per step).  LDS rows are 128 bytes and the
-//     16-byte column index is XORed with row%8, so the row-wise writes and the
-//     32-row fragment reads are both bank-conflict free.
+//     16-byte column index is XORed with (row/2)%8, so the row-wise writes and
+//     the 32-row fragment reads are both bank-conflict free.
 //   - packed weights never touch LDS: a lane of the matrix core's B operand
 //     holds 8 consecutive k of one output column, which is exactly one uint32
 //     of 4-bit codes (two of 8-bit codes).  Each lane streams 128-bit pieces of
@@ -44,7 +44,12 @@ constexpr int kWriteSub = 2;  // sub-step whose fillers publish the next x tile 
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ inline int swz(int row, int chunk) { return row * (BK * 2) + ((chunk ^ (row & 7)) << 4); }
+// LDS has 64 banks of 4 bytes: a 128-bit access is conflict free when every 16
+// consecutive lanes cover one 256-byte window, i.e. two 128-byte rows.  XORing
+// the 16-byte column index with bits 1..3 of the row makes that true both for
+// the row-wise writes (8 lanes per row) and for the fragment reads (16 rows,
+// one column).
+__device__ inline int swz(int row, int chunk) { return row * (BK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 // Per-lane stream of packed weights for the wavefront's two 32-column tiles.
 template <typename T, int GS, int BITS>

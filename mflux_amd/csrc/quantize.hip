@@ -202,10 +202,13 @@ __global__ __launch_bounds__(256) void quantize_kernel(const typename T::storage
 // once per group instead of once per 8 elements, no cross-lane reduction is
 // needed, and scales/biases leave as 128 contiguous bytes per wavefront.
 // LDS slots are XOR-swizzled so that both the row-wise writes and the
-// group-wise reads touch every bank once per 8 lanes.
+// group-wise reads touch every bank once per 16 lanes.
 template <int kChunks>
 __device__ inline int stage_slot(int group, int chunk) {
-  const int f = kChunks >= 8 ? (group & 7) : ((group >> 1) & (kChunks - 1));
+  // 64 banks of 4 bytes: 16 consecutive lanes must cover one 256-byte window.
+  // 8 or 16 pieces per group: two groups / one group per window, XOR with bits
+  // 1..3 of the group; 4 pieces per group: four groups per window, bits 2..3.
+  const int f = kChunks >= 8 ? ((group >> 1) & 7) : ((group >> 2) & (kChunks - 1));
   return group * kChunks + (chunk ^ f);
 }
 

@@ -1,7 +1,7 @@
 """GPU parity: libmfq's quantized matmul (GEMV for M <= 16, MFMA GEMM above)
 against the float64 matmul oracle on MLX-format operands.
 
-Tolerance (BASELINE north star): max |y - y_ref| <= 1e-2 * max|y_ref row|,
+Tolerance of this path: max |y - y_ref| <= 1e-2 * max|y_ref row|,
 per output row.
 """
 import numpy as np
@@ -117,7 +117,7 @@ def test_qmv_one_hot_and_float32_output(oracle):
 
 
 def test_qmv_adaln_config_full(oracle):
-    """BASELINE config 2: SiLU(temb) [M,3072] against W8 [18432,3072]."""
+    """The adaLN modulation shape: SiLU(temb) [M,3072] against W8 [18432,3072]."""
     o = oracle
     for M in (1, 4):
         temb = seeded(2, 0, (M, 3072), 1.0)
@@ -275,7 +275,7 @@ def test_integer_weights_exact(oracle, bits):
 
 @pytest.mark.parametrize("shape", ["linear1", "linear2"])
 def test_qmm_flux_single_block_full_size(oracle, shape):
-    """BASELINE config 3 at full size: sampled rows against the float64 oracle,
+    """The FLUX.1 single-block linears at full size: sampled rows against the float64 oracle,
     and linearity y(x1 + x2) ~ y(x1) + y(x2) on the whole output."""
     import mflux_amd
     from gpu_util import to_dev, u32_to_dev
