@@ -8,20 +8,25 @@
 //
 // Two kernels.
 //
-// qmv_rows_kernel (M <= 4, rows of at most 8 KiB of codes): one wavefront per
+// qmv_rows_kernel (M <= 4, rows of at most 6 KiB of codes): one wavefront per
 // weight row at a time.  The lanes read the row as consecutive 16-byte pieces
 // (lane l takes piece 64*j + l of the row in load j), i.e. every load
 // instruction covers one contiguous KiB, which is the access pattern that
 // reaches HBM speed; loads of the next row are in flight while the current one
-// is consumed.  Each lane dequantises its own codes (one float32 fma per code,
-// single rounding to the 16-bit type) and owns the matching 8-element slices of
-// x, held in registers for the whole kernel.  The dot products run on the
-// 16x16x32 matrix core with BOTH operands indexed by lane: operand A row i /
-// k-block g is lane i+16g's weights, operand B column j / k-block g is lane
-// j+16g's x slice, so the diagonal D[i][i] is the sum over lanes i, i+16,
-// i+32, i+48 of their private dot products, accumulated over all loads of the
-// row.  The 16 diagonal values are summed across the wavefront when the row
-// ends.  The off-diagonal results are never looked at.
+// is consumed.  A lane owns the 8-element slices of x that match its pieces,
+// held in registers for the whole kernel, and a piece lies inside one group.
+// The codes are never converted: one AND-OR per pair of codes turns them into
+// exact 16-bit floats "offset + code" (bfloat16 0x4300 | n = 128 + n for a
+// 4-bit value, 0x4500 | n = 2048 + 16 n for the high half of an 8-bit code;
+// float16 0x6400 | n = 1024 + n), and the 4x4x4 matrix-core instruction, whose
+// 16 independent blocks multiply a lane's four A values with the same lane's
+// four B values on the block diagonal, accumulates sum(x * (offset + code))
+// per lane and piece in float32.  With the lane's sum of x over the piece, Sx,
+//   sum(x * (scale * code + bias)) = scale * D + (bias - offset * scale) * Sx,
+// two float32 fma per piece.  Against dequantising first, this leaves the
+// weights unrounded (closer to exact arithmetic) and takes a quarter of the
+// vector instructions.  The lanes' sums are added across the wavefront when
+// the row ends.
 //
 // qmv_kernel (everything else up to M = 16): a workgroup of four wavefronts
 // owns 16 output features and walks K in phases.  Every lane streams 128-bit
@@ -274,6 +279,36 @@ struct RowRegs {
   }
 };
 
+// Exact 16-bit float images of codes, two per register.
+template <typename T>
+struct CodeFloat;
+template <>
+struct CodeFloat<BF16> {
+  static constexpr uint32_t kNibble = 0x43004300u;      // 128 + n, n < 128
+  static constexpr uint32_t kHighMagic = 0x45004500u;   // 2048 + 16 n
+  static constexpr bool kWholeByte = false;             // 8 significant bits: an 8-bit code goes in as two nibbles
+  static constexpr float kOffset4 = 128.f, kOffset8 = 2048.f + 128.f;
+  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct CodeFloat<F16> {
+  static constexpr uint32_t kNibble = 0x64006400u;  // 1024 + n, n < 1024
+  static constexpr uint32_t kHighMagic = 0;         // unused: a whole byte fits
+  static constexpr bool kWholeByte = true;
+  static constexpr float kOffset4 = 1024.f, kOffset8 = 1024.f;
+  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
+    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+};
+
+// The 4x4x4 instruction: lane l belongs to block l/4 and holds row l%4 of the
+// block's A (4 k values) and column l%4 of its B; result register i of the lane
+// is element (i, l%4) of the block's product, so register l%4 is the dot
+// product of the lane's own A and B values.
 template <typename T, int BITS, int kM, int kMaxLoads, bool kCoop>
 __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq,
                                                        const uint16_t* __restrict__ scales,
@@ -281,17 +316,21 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
                                                        const uint16_t* __restrict__ bias, void* __restrict__ y,
                                                        int y_is_f32, int M, int N, int K, int gs_shift, int rows_per_wave,
                                                        int extra_rows) {
-  using vec8 = typename T::vec8;
   using R = RowRegs<T, BITS, kM, kMaxLoads, kCoop>;
-  constexpr int kCodes = 128 / BITS;  // codes in one 16-byte piece
-  constexpr int kSlots = kCodes / 8;  // matrix-core k slots fed by one piece
+  using CF = CodeFloat<T>;
+  constexpr int kCodes = 128 / BITS;     // codes in one 16-byte piece
+  constexpr int kPerWord = 32 / BITS;    // codes in one 32-bit word
+  constexpr int kXOps = kCodes / 4;      // B operands (4 values of x each) per piece
+  constexpr float kOffset = BITS == 4 ? CF::kOffset4 : CF::kOffset8;
   const int lane = threadIdx.x & (kWave - 1);
   const int row_bytes = K * BITS / 8;
   const int groups = K >> gs_shift;  // the launcher picked kMaxLoads = ceil(row_bytes / 1024)
 
-  // this lane's pieces: position in the row, group, and its slices of x
+  // this lane's pieces: position in the row, group, its slices of x in the
+  // order the code pairs come out of a word, and the sum of each slice
   int piece[kMaxLoads], grp[kMaxLoads];
-  vec8 xf[kM][kMaxLoads][kSlots];
+  uint2 xq[kM][kMaxLoads][kXOps];
+  float sx[kM][kMaxLoads];
 #pragma unroll
   for (int j = 0; j < kMaxLoads; ++j) {
     const int off = (j * kWave + lane) * 16;
@@ -301,16 +340,30 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
     grp[j] = in_row ? (k0 >> gs_shift) : 0;
 #pragma unroll
     for (int m = 0; m < kM; ++m) {
+      float sum = 0.f;
 #pragma unroll
-      for (int h = 0; h < kSlots; ++h) {
-        u32x4 v = {0, 0, 0, 0};
-        if (in_row && m < M) v = *reinterpret_cast<const u32x4*>(x + (int64_t)m * K + k0 + 8 * h);
-        xf[m][j][h] = __builtin_bit_cast(vec8, v);
+      for (int wd = 0; wd < 4; ++wd) {  // the piece's four words
+        if constexpr (BITS == 4) {
+          // word = codes c0..c7; pairs (c0,c4) (c1,c5) | (c2,c6) (c3,c7)
+          u32x4 v = {0, 0, 0, 0};
+          if (in_row && m < M) v = *reinterpret_cast<const u32x4*>(x + (int64_t)m * K + k0 + 8 * wd);
+          xq[m][j][2 * wd] = make_uint2((v[0] & 0xffffu) | (v[2] << 16), (v[0] >> 16) | (v[2] & 0xffff0000u));
+          xq[m][j][2 * wd + 1] = make_uint2((v[1] & 0xffffu) | (v[3] << 16), (v[1] >> 16) | (v[3] & 0xffff0000u));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sum += T::to_f32((uint16_t)v[e]) + T::to_f32((uint16_t)(v[e] >> 16));
+        } else {
+          // word = codes c0..c3; pairs (c0,c2) (c1,c3)
+          uint2 v = {0, 0};
+          if (in_row && m < M) v = *reinterpret_cast<const uint2*>(x + (int64_t)m * K + k0 + 4 * wd);
+          xq[m][j][wd] = make_uint2((v.x & 0xffffu) | (v.y << 16), (v.x >> 16) | (v.y & 0xffff0000u));
+          sum += T::to_f32((uint16_t)v.x) + T::to_f32((uint16_t)(v.x >> 16)) + T::to_f32((uint16_t)v.y) +
+                 T::to_f32((uint16_t)(v.y >> 16));
+        }
       }
+      sx[m][j] = sum;
     }
   }
-  // which of the four result registers holds this lane's diagonal element
-  const int diag = (lane & 15) - 4 * (lane >> 4);
+  static_assert(kPerWord * 4 == kCodes, "a piece is four words");
 
   // rows are dealt to wavefronts in contiguous, balanced runs: rows_per_wave
   // each, one more for the first extra_rows wavefronts (the split is computed
@@ -321,10 +374,20 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
   if (row_begin >= row_end) return;
   const char* wbytes = reinterpret_cast<const char*>(wq);
 
+  // (word & mask) | magic is one instruction when the mask sits in a scalar and
+  // the magic in a vector register; as literals they would cost two.
+  uint32_t pair_mask = (BITS == 8 && CF::kWholeByte) ? 0x00ff00ffu : 0x000f000fu;
+  uint32_t magic = CF::kNibble, magic_high = CF::kHighMagic;
+  asm volatile("" : "+s"(pair_mask), "+v"(magic), "+v"(magic_high));
+
   auto consume = [&](const R& regs, int64_t row) __attribute__((always_inline)) {
-    f32x4 acc[kM], acc_odd[kM];  // two chains per activation row, so that matrix instructions need not wait for each other
+    f32x4 tot[kM];  // register lane%4: this lane's sum of scale * D over its pieces
+    float corr[kM];  // this lane's sum of (bias - offset * scale) * Sx
 #pragma unroll
-    for (int m = 0; m < kM; ++m) acc[m] = acc_odd[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < kM; ++m) {
+      tot[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+      corr[m] = 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < kMaxLoads; ++j) {
       float sc, bi;
@@ -339,28 +402,48 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
         sc = T::to_f32(regs.s[j]);
         bi = T::to_f32(regs.b[j]);
       }
+      // one accumulation chain per piece and activation row; consecutive pieces
+      // are independent of each other
+      f32x4 d[kM];
 #pragma unroll
-      for (int h = 0; h < kSlots; ++h) {
-        uint4 wf;
+      for (int m = 0; m < kM; ++m) d[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd) {
+        const uint32_t w = regs.w[j][wd];
         if constexpr (BITS == 4) {
-          wf = dequant8_w4<T>(regs.w[j][h], sc, bi);
-        } else {
-          wf = dequant8_w8<T>(regs.w[j][2 * h], regs.w[j][2 * h + 1], sc, bi);
-        }
+          const uint2 a0 = make_uint2((w & pair_mask) | magic, ((w >> 4) & pair_mask) | magic);
+          const uint2 a1 = make_uint2(((w >> 8) & pair_mask) | magic, ((w >> 12) & pair_mask) | magic);
 #pragma unroll
-        for (int m = 0; m < kM; ++m) {
-          if (kM == 1 && ((j * kSlots + h) & 1)) {
-            acc_odd[m] = mfma16(__builtin_bit_cast(vec8, wf), xf[m][j][h], acc_odd[m]);
-          } else {
-            acc[m] = mfma16(__builtin_bit_cast(vec8, wf), xf[m][j][h], acc[m]);
+          for (int m = 0; m < kM; ++m) {
+            d[m] = CF::mfma4(a0, xq[m][j][2 * wd], d[m]);
+            d[m] = CF::mfma4(a1, xq[m][j][2 * wd + 1], d[m]);
+          }
+        } else if constexpr (CF::kWholeByte) {
+          const uint2 a = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
+#pragma unroll
+          for (int m = 0; m < kM; ++m) d[m] = CF::mfma4(a, xq[m][j][wd], d[m]);
+        } else {
+          const uint2 lo = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
+          const uint2 hi = make_uint2(((w >> 4) & pair_mask) | magic_high, ((w >> 12) & pair_mask) | magic_high);
+#pragma unroll
+          for (int m = 0; m < kM; ++m) {
+            d[m] = CF::mfma4(lo, xq[m][j][wd], d[m]);
+            d[m] = CF::mfma4(hi, xq[m][j][wd], d[m]);
           }
         }
       }
+      const float bo = __builtin_fmaf(-kOffset, sc, bi);
+#pragma unroll
+      for (int m = 0; m < kM; ++m) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tot[m][e] = __builtin_fmaf(sc, d[m][e], tot[m][e]);
+        corr[m] = __builtin_fmaf(bo, sx[m][j], corr[m]);
+      }
     }
+    const int diag = lane & 3;
 #pragma unroll
     for (int m = 0; m < kM; ++m) {
-      if (kM == 1) acc[m] += acc_odd[m];
-      float v = diag == 0 ? acc[m][0] : diag == 1 ? acc[m][1] : diag == 2 ? acc[m][2] : diag == 3 ? acc[m][3] : 0.f;
+      float v = (diag == 0 ? tot[m][0] : diag == 1 ? tot[m][1] : diag == 2 ? tot[m][2] : tot[m][3]) + corr[m];
       v = wave_sum(v);
       if (lane == 0 && m < M) {
         const int64_t o = (int64_t)m * N + row;
