@@ -114,6 +114,18 @@ __device__ inline uint4 dequant8_w8(uint32_t w0, uint32_t w1, float s, float b) 
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Compute units of the current device (256 on an MI355X).
+inline int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return n;
+}
+
 // Entry points of the individual translation units (host side).
 int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, int bits, uint32_t* wq,
                     void* scales, void* biases, hipStream_t stream);
@@ -131,5 +143,13 @@ int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream);
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
+// the 128 x 128-tile kernel for a few hundred activation rows (K % 64 == 0)
+int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                   const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                   void* workspace, size_t workspace_bytes, hipStream_t stream);
+size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
+// y = sum of `splits` float32 planes of M x N (+ bias), rounded to y's type; dtype is the type of bias and 16-bit y
+int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
+                         int y_dtype, hipStream_t stream);
 
 }  // namespace mfq

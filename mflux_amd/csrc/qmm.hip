@@ -667,17 +667,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 }
 
-int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  }
-  return n;
-}
-
 // ---- K split across workgroups (few tiles, long K) -------------------------
 // With fewer than half as many 256 x 256 tiles as there are CUs, K is cut into
 // `splits` equal ranges of whole periods; range s of every tile is accumulated
@@ -795,14 +784,7 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   if (int rc = launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
                                                 stream))
     return rc;
-  const int64_t plane = M * N;
-  const int64_t threads = (N & 3) == 0 ? plane / 4 : plane;
-  const int64_t blocks = (threads + 255) / 256;
-  const int cap = compute_units() * 8;
-  hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, stream,
-                     (const float*)workspace, plan.splits, plane, (const uint16_t*)bias, (int)N, y,
-                     (int)(y_dtype == MFQ_F32));
-  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+  return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
 }
 
 template <typename T, int GS>
@@ -826,15 +808,46 @@ int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const voi
 
 }  // namespace
 
+// Shapes whose 256 x 256 tiles would leave more than half of the compute units
+// idle go to the 128-column-tile kernel, except many rows against a long K,
+// where cutting K between 256 x 256 tiles measures about a tenth faster.
+inline bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
+  const bool few_tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN) * 2 <= compute_units();
+  return few_tiles && !(M > 512 && K >= 8192);
+}
+
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
   if (K % BK) return 0;
+  if (use_mid_kernel(M, N, K)) return qmm_mid_workspace_bytes(M, N, K, gs);
   const SplitPlan plan = plan_split(M, N, K, period_of(gs), compute_units());
   return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+}
+
+int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
+                         int y_dtype, hipStream_t stream) {
+  const int64_t plane = M * N;
+  const int64_t threads = (N & 3) == 0 ? plane / 4 : plane;
+  const int64_t blocks = (threads + 255) / 256;
+  const int cap = compute_units() * 8;
+  const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+  if (dtype == MFQ_BF16) {
+    hipLaunchKernelGGL((splitk_reduce_kernel<BF16>), grid, dim3(256), 0, stream, (const float*)planes, splits, plane,
+                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32));
+  } else if (dtype == MFQ_F16) {
+    hipLaunchKernelGGL((splitk_reduce_kernel<F16>), grid, dim3(256), 0, stream, (const float*)planes, splits, plane,
+                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32));
+  } else {
+    return MFQ_EDTYPE;
+  }
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (use_mid_kernel(M, N, K))
+    return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
+                          workspace_bytes, stream);
   if (dtype == MFQ_BF16)
     return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
                            stream);

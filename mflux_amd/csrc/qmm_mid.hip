@@ -1,0 +1,503 @@
+// Medium-M W4/W8 x A16 quantized matmul for gfx950 (a few hundred activation
+// rows: the text stream of mflux's joint transformer blocks, e.g.
+// src/mflux/models/flux/model/flux_transformer/joint_transformer_block.py, and
+// the T5 / Qwen text encoders at M = 256..1024):
+//   y[M, N] = x[M, K] @ dequant(wq[N, K])^T (+ bias)
+//
+// With so few rows the 256 x 256 tiles of the large-M kernel are too few to
+// fill the chip, and cutting K to make more of them costs a float32 plane of
+// the output per cut.  Here a workgroup of four wavefronts computes a
+// 128 x 128 tile, two workgroups share a compute unit (two wavefronts per SIMD
+// hide each other's waits, so the code is left to the compiler's scheduler),
+// and K is cut only when even these tiles are too few.
+//   - both operands go through LDS as 16-bit tiles of 128 rows x 64 k, rows of
+//     128 bytes with the 16-byte column index XORed with (row/2)%8: x is copied
+//     (128-bit moves), the weights are dequantised on the way in, every code
+//     exactly once per workgroup (thread t: feature t/2, half t%2 of the 64 k;
+//     one float32 fma per code, single rounding to the 16-bit type);
+//   - global loads run two k steps ahead in registers, the LDS tiles are
+//     double buffered, one barrier per step;
+//   - wavefront (wm, wn) owns rows [64wm, 64wm+64) x columns [64wn, 64wn+64) as
+//     2 x 2 accumulators of the 32x32x16 matrix-core instruction, weights as
+//     the A operand (so a lane ends up with four consecutive output columns).
+#include <type_traits>
+#include <utility>
+
+#include "common.h"
+
+namespace mfq {
+namespace {
+
+constexpr int TN = 128;
+constexpr int TK = 64;
+constexpr int kTileW = TN * TK * 2;  // the 16-bit weight tile: 16 KiB
+// kWavesM wavefronts along M (2 or 4), two along N
+constexpr int tile_m(int waves_m) { return 64 * waves_m; }
+constexpr int threads_of(int waves_m) { return 2 * waves_m * kWave; }
+constexpr int tile_x_bytes(int waves_m) { return tile_m(waves_m) * TK * 2; }
+constexpr int lds_bytes(int waves_m) { return 2 * (tile_x_bytes(waves_m) + kTileW); }  // both tiles, double buffered
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// 64 LDS banks of 4 bytes: a 128-bit access is conflict free when 16
+// consecutive lanes cover one 256-byte window (two rows).
+__device__ inline int swz(int row, int chunk) { return row * (TK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, kN - 1>)
+template <typename F, int... kIs>
+__device__ inline void for_each_index_impl(F&& f, std::integer_sequence<int, kIs...>) {
+  (f(std::integral_constant<int, kIs>{}), ...);
+}
+template <int kN, typename F>
+__device__ inline void for_each_index(F&& f) {
+  for_each_index_impl(f, std::make_integer_sequence<int, kN>{});
+}
+
+template <typename T>
+__device__ inline float lo_f32(uint32_t pk) { return T::to_f32((uint16_t)pk); }
+template <typename T>
+__device__ inline float hi_f32(uint32_t pk) { return T::to_f32((uint16_t)(pk >> 16)); }
+
+// kFast: scales and biases are read as 8-byte pieces (four consecutive groups
+// of a weight row) once per period of 4*GS/64 k steps; otherwise as one 2-byte
+// value per step.
+template <typename T, int GS, int BITS, bool kFast, int kWavesM>
+__global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
+    const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
+    const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
+    int N, int K, int tiles_m, int tiles_n, int steps) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  using vec8 = typename T::vec8;
+  constexpr int TM = tile_m(kWavesM);
+  constexpr int kThreads = threads_of(kWavesM);
+  constexpr int kTileX = tile_x_bytes(kWavesM);
+  constexpr int kBuf = kTileX + kTileW;       // one buffer: the x tile, then the weight tile
+  constexpr int kCodes = TN * TK / kThreads;  // weights a thread dequantises per step: 32 or 16
+  constexpr int kParts = TK / kCodes;         // threads per feature
+  constexpr int kChunks = kCodes / 8;         // 8-code (16-byte) pieces it writes
+  constexpr int kWords = kCodes * BITS / 32;  // 32-bit words of codes it loads
+  constexpr int kPer = 4 * GS / TK;           // k steps covered by one 8-byte scale piece
+  constexpr int kXPass = kThreads / 8;        // x rows copied per pass (four passes)
+
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+  const int wm = wave >> 1, wn = wave & 1;  // wm < kWavesM
+  const int r = lane & 31;
+  const int h = lane >> 5;
+
+  // Work item = (k range, tile).  Workgroups are dealt round-robin to the 8
+  // XCDs; item b is mapped so that an XCD walks a contiguous run of the tile
+  // sequence (tile row fastest), sharing x tiles and weight tiles in its L2.
+  const int n_tiles = tiles_m * tiles_n;
+  const int split = blockIdx.x / n_tiles;
+  int tile = blockIdx.x - split * n_tiles;
+  {
+    const int per_xcd = n_tiles / 8;
+    if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
+  }
+  const int m0 = (tile % tiles_m) * TM;
+  const int n0 = (tile / tiles_m) * TN;
+  const int kb = split * steps * TK;  // first k of the item
+  char* y_item = static_cast<char*>(y) + (size_t)split * M * N * 4;  // split > 0 only with float32 planes
+
+  // global offsets (bytes; they fit 32 bits, checked by the launcher)
+  uint32_t xoff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    xoff[i] = ((uint32_t)min(m0 + (t >> 3) + kXPass * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+  const int f = t / kParts, part = t % kParts;  // this thread's feature of the tile and part of the k step
+  const int hh = part * kCodes / 32;            // which half of the step (the group, for groups of 32)
+  const uint32_t wrow = (uint32_t)min(n0 + f, N - 1);
+  const uint32_t woff = wrow * (uint32_t)(K * BITS / 8) + (uint32_t)(part * kCodes * BITS / 8);
+  const uint32_t soff = wrow * (uint32_t)(K / GS) * 2u;
+  const char* xbytes = reinterpret_cast<const char*>(x);
+  const char* wbytes = reinterpret_cast<const char*>(wq);
+  const char* sbytes = reinterpret_cast<const char*>(scales);
+  const char* bbytes = reinterpret_cast<const char*>(biases);
+
+  // LDS slots
+  const int wr_x = swz(t >> 3, t & 7);
+  int wr_w[kChunks];
+#pragma unroll
+  for (int c = 0; c < kChunks; ++c) wr_w[c] = swz(f, part * kChunks + c);
+  int rd[4];
+#pragma unroll
+  for (int sub = 0; sub < 4; ++sub) rd[sub] = swz(r, 4 * h + sub);
+
+  struct Stage {
+    u32x4 x[4];
+    uint32_t w[kWords];
+    uint16_t s, b;  // !kFast
+  };
+  struct Period {  // kFast: scales and biases of four consecutive groups of the thread's weight row
+    uint2 s, b;
+  };
+  Stage st[2];
+  Period per[2];  // periods with an even / odd index
+
+  // Everything below is unconditional and its register sets are chosen at
+  // compile time, so that every wait for a load can leave exactly the younger
+  // loads in flight.  q: k step inside the item (steps past the end repeat the
+  // last one and are never consumed).
+  // sel: -1, or the Period set to refill with the period that step q starts.
+  auto load = [&](auto sel, Stage& g, int q) __attribute__((always_inline)) {
+    constexpr int kSel = decltype(sel)::value;
+    const int k0 = kb + min(q, steps - 1) * TK;
+    // in the order publishing consumes them
+    if constexpr (kFast) {
+      if constexpr (kSel >= 0) {
+        const int g0 = (k0 / GS) & ~3;
+        per[kSel].s = *reinterpret_cast<const uint2*>(sbytes + soff + (size_t)g0 * 2);
+        per[kSel].b = *reinterpret_cast<const uint2*>(bbytes + soff + (size_t)g0 * 2);
+      }
+    } else {
+      const int g0 = k0 / GS + (GS == 32 ? hh : 0);
+      g.s = *reinterpret_cast<const uint16_t*>(sbytes + soff + (size_t)g0 * 2);
+      g.b = *reinterpret_cast<const uint16_t*>(bbytes + soff + (size_t)g0 * 2);
+    }
+    const char* wsrc = wbytes + (size_t)k0 * BITS / 8 + woff;
+    if constexpr (kWords == 2) {
+      const uint2 v = *reinterpret_cast<const uint2*>(wsrc);
+      g.w[0] = v.x;
+      g.w[1] = v.y;
+    } else {
+#pragma unroll
+      for (int l = 0; l < kWords / 4; ++l) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(wsrc + 16 * l);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) g.w[4 * l + e] = v[e];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) g.x[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k0 * 2 + xoff[i]);
+  };
+  // the Period set step e of the unrolled sequence refills, if it starts a period
+  auto sel_of = [](auto e) {
+    constexpr int kE = decltype(e)::value % (2 * kPer);
+    return std::integral_constant<int, (kFast && kE % kPer == 0) ? kE / kPer : -1>{};
+  };
+
+  // Scale and bias of this thread's 32 codes in step e of the unrolled sequence.
+  auto scale_of = [&](auto e, const Stage& g, float& sc, float& bi) __attribute__((always_inline)) {
+    if constexpr (kFast) {
+      constexpr int kE = decltype(e)::value % (2 * kPer);
+      constexpr int kIn = kE % kPer;
+      const int idx = GS >= TK ? kIn * TK / GS : 2 * kIn + hh;  // group inside the period
+      const Period& pr = per[kE / kPer];
+      sc = T::to_f32((uint16_t)((((uint64_t)pr.s.y << 32) | pr.s.x) >> (16 * idx)));
+      bi = T::to_f32((uint16_t)((((uint64_t)pr.b.y << 32) | pr.b.x) >> (16 * idx)));
+    } else {
+      sc = T::to_f32(g.s);
+      bi = T::to_f32(g.b);
+    }
+  };
+  // Quarter c of publishing a step's registers to buffer `buf`: one 128-bit
+  // piece of x and (in every quarter, or every other one) eight dequantised
+  // weights.
+  auto publish_part = [&](const Stage& g, int c, float sc, float bi, int buf) __attribute__((always_inline)) {
+    char* xd = lds + buf * kBuf;
+    char* wd = xd + kTileX;
+    *reinterpret_cast<u32x4*>(xd + wr_x + kXPass * TK * 2 * c) = g.x[c];
+    constexpr int kEvery = 4 / kChunks;
+    if (c % kEvery == 0) {
+      const int cw = c / kEvery;
+      uint4 v;
+      if constexpr (BITS == 4) {
+        v = dequant8_w4<T>(g.w[cw], sc, bi);
+      } else {
+        v = dequant8_w8<T>(g.w[2 * cw], g.w[2 * cw + 1], sc, bi);
+      }
+      *reinterpret_cast<uint4*>(wd + wr_w[cw]) = v;
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // Step e of the unrolled sequence, k step p of the item: the matrix work on
+  // buffer e%2, with quarter `sub` of publishing step p+1 to the other buffer
+  // in the shadow of the matrix instructions of sub-step `sub` (a scheduling
+  // barrier between sub-steps keeps the interleaving), then the loads of step
+  // p+3 into the registers just published.
+  auto step = [&](auto e, int p) __attribute__((always_inline)) {
+    constexpr int kE = decltype(e)::value;
+    constexpr int buf = kE & 1;
+    const Stage& next = st[buf ^ 1];
+    const char* xs = lds + buf * kBuf + 4096 * (2 * wm);
+    const char* ws = lds + buf * kBuf + kTileX + 4096 * (2 * wn);
+    float sc, bi;
+    scale_of(std::integral_constant<int, kE + 1>{}, next, sc, bi);
+    vec8 af[2][2], bf[2][2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) af[0][j] = *reinterpret_cast<const vec8*>(ws + rd[0] + 4096 * j);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) bf[0][i] = *reinterpret_cast<const vec8*>(xs + rd[0] + 4096 * i);
+#pragma unroll
+    for (int sub = 0; sub < 4; ++sub) {
+      if (sub < 3) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) af[(sub + 1) & 1][j] = *reinterpret_cast<const vec8*>(ws + rd[sub + 1] + 4096 * j);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) bf[(sub + 1) & 1][i] = *reinterpret_cast<const vec8*>(xs + rd[sub + 1] + 4096 * i);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(af[sub & 1][j], bf[sub & 1][i], acc[i][j]);
+      publish_part(next, sub, sc, bi, buf ^ 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    load(sel_of(std::integral_constant<int, kE + 3>{}), st[buf ^ 1], p + 3);
+    __syncthreads();
+  };
+
+  // prologue: steps 0, 1, 2 in flight, step 0 published
+  {
+    const std::integral_constant<int, 0> e0{};
+    load(sel_of(e0), st[0], 0);
+    load(sel_of(std::integral_constant<int, 1>{}), st[1], 1);
+    float sc, bi;
+    scale_of(e0, st[0], sc, bi);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) publish_part(st[0], c, sc, bi, 0);
+    load(sel_of(std::integral_constant<int, 2>{}), st[0], 2);
+    __syncthreads();
+  }
+  // The sequence is unrolled over two scale periods (kFast) or two steps.
+  constexpr int kSeq = kFast ? 2 * kPer : 2;
+  int p = 0;
+  for (; p + kSeq <= steps; p += kSeq) for_each_index<kSeq>([&](auto e) __attribute__((always_inline)) { step(e, p + decltype(e)::value); });
+  if constexpr (kFast) {
+    // whole periods: what remains is one period
+    if (p < steps) for_each_index<kPer>([&](auto e) __attribute__((always_inline)) { step(e, p + decltype(e)::value); });
+  } else {
+    if (p < steps) step(std::integral_constant<int, 0>{}, p);
+  }
+
+  // ---- epilogue: accumulator [i][j], register e holds output row
+  // m0 + 64wm + 32i + r and column n0 + 64wn + 32j + 8(e/4) + 4h + e%4.
+  // Every LDS tile is free now (the loop ended with a barrier); each wavefront
+  // transposes its block through a private region so that a global store
+  // instruction writes whole row segments.
+  const int mw = m0 + 64 * wm, nw = n0 + 64 * wn;
+  if (!y_is_f32 && (N & 7) == 0) {
+    constexpr int kStride = 144;  // 64 16-bit columns + 16 bytes of padding
+    char* stage = lds + wave * (64 * kStride);
+    uint16_t* yout = reinterpret_cast<uint16_t*>(y_item);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) {
+        const int cl = 32 * j + 8 * eb + 4 * h;
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(nw + cl + c, N - 1)]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          uint32_t pk[2];
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            pk[c] = T::pack2(acc[i][j][4 * eb + 2 * c], acc[i][j][4 * eb + 2 * c + 1]);
+            if (bias)  // second rounding, as a separate add on the 16-bit result would do
+              pk[c] = T::pack2(lo_f32<T>(pk[c]) + bv[2 * c], hi_f32<T>(pk[c]) + bv[2 * c + 1]);
+          }
+          *reinterpret_cast<uint2*>(stage + (32 * i + r) * kStride + cl * 2) = make_uint2(pk[0], pk[1]);
+        }
+      }
+    }
+    const int cg = nw + 8 * (lane & 7);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int rl = 8 * k + (lane >> 3);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 16 * (lane & 7));
+      const int row = mw + rl;
+      if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
+    }
+  } else if (y_is_f32 && (N & 3) == 0) {
+    constexpr int kStride = 64 * 4 + 16;
+    char* stage = lds + wave * (32 * kStride);
+    float* yout = reinterpret_cast<float*>(y_item);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int eb = 0; eb < 4; ++eb) {
+          const int cl = 32 * j + 8 * eb + 4 * h;
+          float bv[4] = {0.f, 0.f, 0.f, 0.f};
+          if (bias) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(nw + cl + c, N - 1)]);
+          }
+          *reinterpret_cast<float4*>(stage + r * kStride + cl * 4) =
+              make_float4(acc[i][j][4 * eb] + bv[0], acc[i][j][4 * eb + 1] + bv[1], acc[i][j][4 * eb + 2] + bv[2],
+                          acc[i][j][4 * eb + 3] + bv[3]);
+        }
+      }
+      const int cg = nw + 4 * (lane & 15);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int rl = 4 * k + (lane >> 4);
+        const float4 v = *reinterpret_cast<const float4*>(stage + rl * kStride + 16 * (lane & 15));
+        const int row = mw + 32 * i + rl;
+        if (row < M && cg < N) *reinterpret_cast<float4*>(yout + (int64_t)row * N + cg) = v;
+      }
+    }
+  } else {
+    // any N: element-wise guarded stores straight from the accumulators
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int eb = 0; eb < 4; ++eb) {
+        const int col = nw + 32 * j + 8 * eb + 4 * h;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int row = mw + 32 * i + r;
+          if (row >= M) continue;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            if (col + c >= N) continue;
+            const float bv = bias ? T::to_f32(bias[col + c]) : 0.f;
+            const int64_t o = (int64_t)row * N + col + c;
+            if (y_is_f32) {
+              reinterpret_cast<float*>(y_item)[o] = acc[i][j][4 * eb + c] + bv;
+            } else {
+              uint16_t hv = T::from_f32(acc[i][j][4 * eb + c]);
+              if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
+              reinterpret_cast<uint16_t*>(y_item)[o] = hv;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+struct MidPlan {
+  int splits;
+  int steps;  // k steps per range
+};
+
+inline int period_of(int gs) { return 4 * gs / TK; }
+
+// Up to 128 activation rows: 128-row tiles, two workgroups of four wavefronts
+// per compute unit.  More: 256-row tiles (every dequantised weight then serves
+// twice the matrix work), one workgroup of eight wavefronts per compute unit.
+inline int waves_m_of(int64_t M) { return M <= 128 ? 2 : 4; }
+
+// K is cut into equal ranges of whole scale periods (at least 8 k steps each)
+// while the work items are fewer than the compute units and the cut keeps them
+// within what runs at once.
+inline MidPlan plan_mid(int64_t M, int64_t N, int64_t K, int period, int cus) {
+  const int steps = (int)(K / TK);
+  const int waves_m = waves_m_of(M);
+  const int tm = tile_m(waves_m);
+  const int64_t tiles = ((M + tm - 1) / tm) * ((N + TN - 1) / TN);
+  const int64_t slots = waves_m == 2 ? 2 * (int64_t)cus : cus;
+  MidPlan plan{1, steps};
+  if (steps % period != 0) return plan;
+  for (int s = 2; s <= steps / 8 && tiles * plan.splits < cus && tiles * s <= slots; ++s)
+    if (steps % s == 0 && (steps / s) % period == 0) plan = MidPlan{s, steps / s};
+  return plan;
+}
+
+template <typename T, int GS, int BITS, bool kFast, int kWavesM>
+int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                  const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream) {
+  auto kernel = qmm_mid_kernel<T, GS, BITS, kFast, kWavesM>;
+  constexpr int kLds = lds_bytes(kWavesM);
+  static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kLds) != hipSuccess)
+      return MFQ_ELAUNCH;
+    configured = true;
+  }
+  const int tiles_m = (int)((M + tile_m(kWavesM) - 1) / tile_m(kWavesM));
+  const int tiles_n = (int)((N + TN - 1) / TN);
+  const int64_t n_items = (int64_t)tiles_m * tiles_n * plan.splits;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)n_items), dim3(threads_of(kWavesM)), kLds, stream, (const uint16_t*)x, wq,
+                     (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.steps);
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T, int GS, int BITS, bool kFast>
+int launch_tile(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream) {
+  if (waves_m_of(M) == 2)
+    return launch_kernel<T, GS, BITS, kFast, 2>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream);
+  return launch_kernel<T, GS, BITS, kFast, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream);
+}
+
+template <typename T, int GS, int BITS>
+int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+               const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
+               hipStream_t stream) {
+  const int64_t steps = K / TK;
+  constexpr int kPer = 4 * GS / TK;
+  const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
+  if (!(steps % kPer == 0 && aligned8))
+    return launch_tile<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
+                                           stream);
+  const MidPlan plan = plan_mid(M, N, K, kPer, compute_units());
+  const size_t need = (size_t)plan.splits * M * N * sizeof(float);
+  if (plan.splits == 1 || !workspace || workspace_bytes < need || !aligned16(workspace))
+    return launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
+                                          stream);
+  if (int rc = launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
+                                              stream))
+    return rc;
+  return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
+}
+
+template <typename T, int GS>
+int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
+                hipStream_t stream) {
+  if (bits == 4) return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
+}
+
+template <typename T>
+int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+              const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
+              hipStream_t stream) {
+  switch (gs) {
+    case 32: return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    case 64: return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    default: return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+  }
+}
+
+}  // namespace
+
+size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
+  if (K % TK) return 0;
+  const MidPlan plan = plan_mid(M, N, K, period_of(gs), compute_units());
+  return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+}
+
+int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                   const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                   void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  // 32-bit byte offsets into x, the packed weight and the scales
+  if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
+  if (dtype == MFQ_BF16)
+    return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                           stream);
+  if (dtype == MFQ_F16)
+    return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                          stream);
+  return MFQ_EDTYPE;
+}
+
+}  // namespace mfq

@@ -481,17 +481,6 @@ __global__ __launch_bounds__(256) void qmv_rows_kernel(const uint16_t* __restric
   }
 }
 
-int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  }
-  return n;
-}
-
 template <typename T, int BITS, int kM, int kMaxLoads, bool kCoop>
 int launch_rows_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                        const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {

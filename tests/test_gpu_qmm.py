@@ -342,21 +342,68 @@ def test_leading_batch_dims_and_dtype_promotion():
     assert float((y32 - y16.float()).abs().max()) < 0.05
 
 
-def test_f16_path(oracle):
+@pytest.mark.parametrize("bits", [4, 8])
+def test_f16_path(oracle, bits):
+    """float16 activations, scales and biases: one activation row (codes enter
+    the matrix core as 1024 + code), a few rows, both tile heights of the
+    medium-M kernel (with and without a K split) and the large-M kernel."""
     import mflux_amd
     from gpu_util import raw
 
     o = oracle
     torch.manual_seed(2)
-    for M in (3, 300):
-        x = torch.randn(M, 512, device="cuda").to(torch.float16)
-        w = (torch.randn(192, 512, device="cuda") * 0.02).to(torch.float16)
-        wq, s, b = mflux_amd.quantize(w, 64, 8)
-        e = o.c_quantize(raw(w), o.F16, 64, 8)
+    for M, K, N in ((1, 3072, 200), (3, 512, 192), (100, 512, 192), (300, 2048, 192), (1100, 512, 4200)):
+        x = torch.randn(M, K, device="cuda").to(torch.float16)
+        w = (torch.randn(N, K, device="cuda") * 0.02).to(torch.float16)
+        wq, s, b = mflux_amd.quantize(w, 64, bits)
+        e = o.c_quantize(raw(w), o.F16, 64, bits)
         assert np.array_equal(raw(wq), e[0])
-        y = mflux_amd.quantized_matmul(x, wq, s, b, bits=8)
-        ref = o.quantized_matmul_f64(x.double().cpu().numpy(), raw(wq), raw(s), raw(b), o.F16, 64, 8)
+        y = mflux_amd.quantized_matmul(x, wq, s, b, bits=bits)
+        ref = o.quantized_matmul_f64(x.double().cpu().numpy(), raw(wq), raw(s), raw(b), o.F16, 64, bits)
         _assert_close(y, ref)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 32), (8, 32), (4, 128), (8, 128)])
+@pytest.mark.parametrize("M,K,N", [(100, 512, 1000), (128, 3072, 136), (129, 1024, 264), (256, 2048, 520),
+                                   (400, 768, 130), (77, 768, 3072)])
+def test_qmm_medium_m(oracle, bits, gs, M, K, N):
+    """The 128-column-tile kernel: 128-row tiles (M <= 128) and 256-row tiles,
+    ragged M and N, K with and without a split, a K that is not a whole number
+    of scale periods (768 with groups of 128), all group sizes; bf16 with bias
+    and float32 output."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    args = _case(o, 31, M, K, N, bits, gs=gs)
+    ref = _ref(o, *args, bits, gs)
+    _assert_close(_run(o, *args, bits, gs), ref)
+    x, wq, s, b, bias = args
+    y32 = mflux_amd.quantized_matmul(to_dev(x, o.BF16).float(), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                     group_size=gs, bits=bits, bias=to_dev(bias, o.BF16))
+    assert y32.dtype == torch.float32
+    _assert_close(y32, ref, tol=5e-3)
+
+
+def test_qmm_medium_m_odd_n(oracle):
+    """N not a multiple of 4: element-wise guarded stores."""
+    o = oracle
+    for M, N in ((90, 131), (300, 77)):
+        args = _case(o, 32, M, 512, N, 4)
+        _assert_close(_run(o, *args, 4), _ref(o, *args, 4))
+
+
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 128)])
+def test_qmm_many_rows_long_k_split(oracle, bits, gs):
+    """More than 512 rows, few 256 x 256 tiles and K >= 8192: the large-M
+    kernel with K cut across compute units."""
+    from mflux_amd import _lib
+
+    o = oracle
+    M, K, N = 600, 8192, 256
+    assert _lib.load().mfq_qmm_t_workspace_bytes(M, K, N, gs, bits) >= 2 * M * N * 4
+    args = _case(o, 33, M, K, N, bits, gs=gs)
+    _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs))
 
 
 @pytest.mark.parametrize("bits", [4, 8, 5])
