@@ -11,10 +11,13 @@ operands resident in HBM.
 The same line carries
   roofline     - the W4A16 GEMM kernel against the dense bf16 MFMA peak, from
                  HIP-event timing of the launches in the timed region;
-  secondary    - the W8 dequant-GEMV (adaLN modulation shape, M=1 and M=4) against
-                 the HBM peak, weights rotated through > 256 MB so the memory-
-                 side cache cannot serve them, and the quantize/pack pass over
-                 both block weights;
+  secondary    - the W8 (and W4) dequant-GEMV (adaLN modulation shape, M=1 and
+                 M=4) against the HBM peak, weights rotated through > 256 MB so
+                 the memory-side cache cannot serve them; the quantize/pack
+                 pass over both block weights; the text-stream shapes (M=512)
+                 of a joint block; and, for comparison, the BLAS library's
+                 plain bf16 GEMM on the step's own activations and dequantised
+                 weights;
   cpu_baseline - the CPU oracle's scalar qmm (a port of MLX's CPU loop; MLX
                  itself cannot be installed here) on a bounded row sample.
 """
@@ -222,33 +225,58 @@ def main():
         K, N = x.shape[1], wq.shape[0]
         per_shape[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
 
-    # ---- secondary: W8 GEMV (config 2), cold weights ---------------------------
+    # ---- secondary: the library's bf16 GEMM on the same operands ---------------
+    library = {}
+    for name, x, wq, s, b in (() if args.no_secondary else ops):
+        w16 = mflux_amd.dequantize(wq, s, b, group_size=GS, bits=BITS)
+        for _ in range(5):  # the library picks and caches its kernel on the first calls
+            torch.matmul(x, w16.t())
+        torch.cuda.synchronize()
+        ms = event_ms(lambda: torch.matmul(x, w16.t()), 20, torch)
+        K, N = x.shape[1], wq.shape[0]
+        library[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
+        del w16
+
+    # ---- secondary: GEMV of the adaLN modulation shape, cold weights -----------
     gemv = {}
     Kg, Ng = 3072, 18432
-    n_buf = 0 if args.no_secondary else 8
-    bufs = []
-    for i in range(n_buf):
-        w = (torch.randn(Ng, Kg, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
-        bufs.append(mflux_amd.quantize(w, GS, 8))
+    for bits_g in (() if args.no_secondary else (8, 4)):
+        n_buf = 8 if bits_g == 8 else 16  # more than 256 MB in rotation
+        bufs = []
+        for i in range(n_buf):
+            w = (torch.randn(Ng, Kg, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+            bufs.append(mflux_amd.quantize(w, GS, bits_g))
+            del w
+        bias = (torch.randn(Ng, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        res = {}
+        for Mg in (1, 4):
+            temb = torch.randn(Mg, Kg, device=dev, generator=gen)
+            xg = torch.nn.functional.silu(temb).to(torch.bfloat16)
+            state = {"i": 0}
+
+            def gemv_call():
+                wqg, sg, bg = bufs[state["i"] % n_buf]
+                state["i"] += 1
+                mflux_amd.quantized_matmul(xg, wqg, sg, bg, group_size=GS, bits=bits_g, bias=bias)
+
+            ms = graph_ms(gemv_call, 4 * n_buf, 10, torch)
+            nbytes = qmm_bytes(Mg, Kg, Ng, bits_g, bias=True)
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            res[f"M{Mg}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                             "bytes": nbytes,
+                             "weights": f"rotating over {n_buf} buffers ({n_buf * Ng * Kg * bits_g // 8 >> 20} MiB)"}
+        gemv[f"w{bits_g}"] = res
+        del bufs
+
+    # ---- secondary: the text stream of a joint block (M = 512) -----------------
+    medium = {}
+    for (Km, Nm) in (() if args.no_secondary else ((3072, 3072), (3072, 12288), (12288, 3072))):
+        xm = torch.randn(512, Km, device=dev, generator=gen).to(torch.bfloat16)
+        w = (torch.randn(Nm, Km, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        wqm, sm, bm = mflux_amd.quantize(w, GS, BITS)
         del w
-    bias = (torch.randn(Ng, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
-    for Mg in (() if args.no_secondary else (1, 4)):
-        temb = torch.randn(Mg, Kg, device=dev, generator=gen)
-        xg = torch.nn.functional.silu(temb).to(torch.bfloat16)
-        state = {"i": 0}
-
-        def gemv_call():
-            wq8, s8, b8 = bufs[state["i"] % n_buf]
-            state["i"] += 1
-            mflux_amd.quantized_matmul(xg, wq8, s8, b8, group_size=GS, bits=8, bias=bias)
-
-        state["i"] = 0
-        ms = graph_ms(gemv_call, 4 * n_buf, 10, torch)
-        nbytes = qmm_bytes(Mg, Kg, Ng, 8, bias=True)
-        gbs = nbytes / (ms * 1e-3) / 1e9
-        gemv[f"M{Mg}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
-                          "bytes": nbytes, "weights": f"rotating over {n_buf} buffers ({n_buf * Ng * Kg >> 20} MiB)"}
-    del bufs
+        ms = graph_ms(lambda: mflux_amd.quantized_matmul(xm, wqm, sm, bm, group_size=GS, bits=BITS), 10, 5, torch)
+        medium[f"{Km}x{Nm}"] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * 512 * Km * Nm / ms / 1e9, 1)}
 
     quant = {}
     for (name, K, N) in (() if args.no_secondary else LINEARS):
@@ -274,8 +302,9 @@ def main():
                    "M": M_TOKENS, "bits": BITS, "group_size": GS},
         "roofline": roofline,
         "per_shape": per_shape,
-        "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "gemv_w8": gemv,
-                      "quantize_w4": quant},
+        "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "gemv_w8": gemv.get("w8", {}),
+                      "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
+                      "library_bf16_gemm_same_operands": library},
     }
     if not args.no_cpu_baseline:
         name, x, wq, s, b = ops[0]
