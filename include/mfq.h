@@ -119,8 +119,12 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
  *   biases  [N, K/group_size]      sb_dtype
  *   bias    [N] or NULL            sb_dtype
  *   y       [M, N]                 y_dtype (sb_dtype or MFQ_F32)
- * M <= 16 runs the HBM-bound dequant-GEMV kernel, larger M the MFMA GEMM.
- * Accumulation is float32 throughout.
+ * M <= 16 runs the HBM-bound dequant-GEMV kernel, larger M one of two MFMA
+ * GEMM kernels (128-column tiles while 256 x 256 tiles would leave more than
+ * half of the compute units idle, 256 x 256 tiles otherwise).  Accumulation is
+ * float32 throughout.  For M > 1 the dequantised weights are rounded once to
+ * x_dtype; for M = 1 x is multiplied with the raw codes and scale and bias are
+ * applied to the float32 sums.
  */
 int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
               const uint32_t* wq, const void* scales, const void* biases,
@@ -129,11 +133,11 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
 
 /*
  * mfq_qmm_t with an optional float32 workspace.  Has no counterpart in the
- * reference (MLX allocates inside its ops).  Shapes with far fewer 256 x 256
- * output tiles than the GPU has compute units -- the text-stream linears of the
- * double blocks, M = 256 or 512 tokens against N = 3072, e.g.
+ * reference (MLX allocates inside its ops).  Shapes with fewer output tiles
+ * than the GPU has compute units -- the text-stream linears of the double
+ * blocks, M = 256 or 512 tokens against N = 3072, e.g.
  * src/mflux/models/qwen/model/qwen_transformer/qwen_transformer_block.py:36-37
- * on the caption tokens -- leave most of the chip idle; with a workspace K is
+ * on the caption tokens -- leave part of the chip idle; with a workspace K is
  * cut into ranges that run on different compute units, each range accumulates
  * into its own float32 plane of the workspace, and a second kernel adds the
  * planes, rounds and applies the bias (same two roundings as the fused
