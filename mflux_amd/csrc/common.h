@@ -112,6 +112,32 @@ __device__ inline uint4 dequant8_w8(uint32_t w0, uint32_t w1, float s, float b) 
   return r;
 }
 
+// Exact 16-bit float images of codes, two per register.
+template <typename T>
+struct CodeFloat;
+template <>
+struct CodeFloat<BF16> {
+  static constexpr uint32_t kNibble = 0x43004300u;      // 128 + n, n < 128
+  static constexpr uint32_t kHighMagic = 0x45004500u;   // 2048 + 16 n
+  static constexpr bool kWholeByte = false;             // 8 significant bits: an 8-bit code goes in as two nibbles
+  static constexpr float kOffset4 = 128.f, kOffset8 = 2048.f + 128.f;
+  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct CodeFloat<F16> {
+  static constexpr uint32_t kNibble = 0x64006400u;  // 1024 + n, n < 1024
+  static constexpr uint32_t kHighMagic = 0;         // unused: a whole byte fits
+  static constexpr bool kWholeByte = true;
+  static constexpr float kOffset4 = 1024.f, kOffset8 = 1024.f;
+  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
+    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+};
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Compute units of the current device (256 on an MI355X).
@@ -137,6 +163,12 @@ int launch_dequantize_rows(const uint32_t* wq, const void* scales, const void* b
 int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream);
+// four weight rows at a time, M <= 4 (qmv_quad_covers() says whether it takes a shape)
+bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* scales, const void* biases,
+                     const void* y, int y_dtype);
+int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                    hipStream_t stream);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,

@@ -6,7 +6,8 @@
 // one or a few activation rows against a wide weight, so the kernel is bound
 // by streaming the packed weight from HBM once.
 //
-// Two kernels.
+// Two kernels here; a third, for two to four activation rows, is in
+// qmv_quad.hip.
 //
 // qmv_rows_kernel (M <= 4, rows of at most 6 KiB of codes): one wavefront per
 // weight row at a time.  The lanes read the row as consecutive 16-byte pieces
@@ -276,32 +277,6 @@ struct RowRegs {
       }
     }
     bias = bias_v ? bias_v[row] : (uint16_t)0;
-  }
-};
-
-// Exact 16-bit float images of codes, two per register.
-template <typename T>
-struct CodeFloat;
-template <>
-struct CodeFloat<BF16> {
-  static constexpr uint32_t kNibble = 0x43004300u;      // 128 + n, n < 128
-  static constexpr uint32_t kHighMagic = 0x45004500u;   // 2048 + 16 n
-  static constexpr bool kWholeByte = false;             // 8 significant bits: an 8-bit code goes in as two nibbles
-  static constexpr float kOffset4 = 128.f, kOffset8 = 2048.f + 128.f;
-  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
-    typedef short s16x4 __attribute__((ext_vector_type(4)));
-    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
-  }
-};
-template <>
-struct CodeFloat<F16> {
-  static constexpr uint32_t kNibble = 0x64006400u;  // 1024 + n, n < 1024
-  static constexpr uint32_t kHighMagic = 0;         // unused: a whole byte fits
-  static constexpr bool kWholeByte = true;
-  static constexpr float kOffset4 = 1024.f, kOffset8 = 1024.f;
-  __device__ static inline f32x4 mfma4(uint2 a, uint2 b, f32x4 c) {
-    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
   }
 };
 
@@ -611,6 +586,10 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream) {
   if (M > kRowsPerBlock) return MFQ_EUNSUPPORTED;
+  // two to four activation rows: four weight rows at a time (for a single row
+  // the one-row-per-wavefront kernel below is the faster of the two)
+  if (M >= 2 && qmv_quad_covers(M, K, N, gs, bits, scales, biases, y, y_dtype))
+    return launch_qmv_quad(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   if (rows_kernel_covers(M, K, bits)) {
     if (dtype == MFQ_BF16)
       return launch_rows<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);

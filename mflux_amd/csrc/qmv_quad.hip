@@ -1,0 +1,351 @@
+// Quantized matvec for one to four activation rows on gfx950, four weight rows
+// at a time: y[0:M, n] = x[0:M] . dequant(W[n]) (+ bias), M <= 4.  The adaLN
+// modulation shape of mflux's transformer blocks
+// (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12).
+//
+// The 4x4x4 matrix-core instruction computes 16 independent 4x4 products: lane
+// l belongs to block l/4 and holds row l%4 of the block's A (4 k values) and
+// column l%4 of its B; register i of lane (b, j) receives element (i, j).  Here
+// a wavefront works on four consecutive weight rows r0..r0+3: block b covers
+// 16-byte piece 16*load + b of each row, lane (b, i) holds that piece of row
+// r0+i as A and the matching slice of activation row i as B.  All 16 results of
+// a block are useful: register i of lane (b, j) accumulates row r0+i against
+// activation row j, so up to four activation rows cost what one does, and every
+// load instruction reads 256 contiguous bytes of each of four adjacent rows.
+//   - codes are not converted: one AND-OR per pair of codes makes the exact
+//     16-bit floats "offset + code" (see CodeFloat), the matrix core sums
+//     x * (offset + code) per piece in float32 (a piece lies in one group), and
+//     scale * D + (bias - offset * scale) * sum(x) is the piece's contribution;
+//     scale and bias of row r0+i reach the other lanes of the block as DPP
+//     quad broadcasts;
+//   - the B operands (x, permuted to the order the code pairs come out of a
+//     word) sit in LDS for the whole kernel, one conflict-free 512-byte line per
+//     operand; the scales and biases of the next four rows are fetched with one
+//     16-byte load per lane and staged through a wavefront-private LDS region;
+//   - weight loads run kRing pieces ahead in a ring of registers, across row
+//     quads; all of them are unconditional (past the end: the wavefront's last
+//     quad again) so that waits can leave exactly the younger loads in flight;
+//   - the 16 blocks' sums are added with two DPP row rotations and two
+//     ds_bpermute exchanges per result register.
+#include <type_traits>
+#include <utility>
+
+#include "common.h"
+
+namespace mfq {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kDppRowRor4 = 0x124;
+constexpr int kDppRowRor8 = 0x128;
+
+template <int kCtrl>
+__device__ inline float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xf, 0xf, false));
+}
+
+template <typename F, int... kIs>
+__device__ inline void for_each_index_impl(F&& f, std::integer_sequence<int, kIs...>) {
+  (f(std::integral_constant<int, kIs>{}), ...);
+}
+template <int kN, typename F>
+__device__ inline void for_each_index(F&& f) {
+  for_each_index_impl(f, std::make_integer_sequence<int, kN>{});
+}
+
+constexpr int kScaleRegion = 1024;  // per wavefront and buffer: 512 bytes of scales, 512 of biases
+
+// kLoads: 256-byte pieces per weight row (K * BITS / 8 / 256); kRing divides it.
+template <typename T, int BITS, int kLoads, int kRing>
+__global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq,
+                                                       const uint16_t* __restrict__ scales,
+                                                       const uint16_t* __restrict__ biases,
+                                                       const uint16_t* __restrict__ bias, void* __restrict__ y,
+                                                       int y_is_f32, int M, int N, int K, int gs_shift,
+                                                       int quads_per_wave) {
+  using CF = CodeFloat<T>;
+  constexpr int kCodes = 128 / BITS;  // codes in one 16-byte piece
+  constexpr int kXOps = kCodes / 4;   // B operands (4 values of x) per piece
+  constexpr float kOffset = BITS == 4 ? CF::kOffset4 : CF::kOffset8;
+  constexpr int kXBytes = kLoads * kXOps * 512;  // the B operands of one lane set
+  static_assert(kLoads % kRing == 0, "ring slots must be known at compile time");
+  extern __shared__ __attribute__((aligned(16))) char lds[];  // x operands, slice sums, 4 x 2 scale regions
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int blk = lane >> 2, li = lane & 3;
+  const int row_bytes = kLoads * 256;
+  const int groups = K >> gs_shift;
+
+  // quads of rows are dealt to wavefronts in contiguous runs of equal length
+  // (the host sizes the grid for that; only the last run can be short or empty)
+  const int wave_id = blockIdx.x * (blockDim.x / kWave) + wave;
+  const int q_begin = wave_id * quads_per_wave;
+  const int q_end = min(q_begin + quads_per_wave, N / 4);
+  const bool has_work = q_begin < q_end;
+
+  char* sreg = lds + kXBytes + kLoads * 256 + wave * 2 * kScaleRegion;  // this wavefront's two scale regions
+  const char* wbytes = reinterpret_cast<const char*>(wq);
+  // this lane's byte offset inside a quad's weights: row li, piece blk
+  const uint32_t lane_woff = (uint32_t)li * (uint32_t)row_bytes + (uint32_t)blk * 16u;
+  // scale fetch: lanes 0..31 take 16 bytes of the quad's scales, lanes 32..63 of its biases
+  const int quad_sb_bytes = 8 * groups;  // four rows of one array
+  const char* sb_src = reinterpret_cast<const char*>(lane < 32 ? scales : biases);
+  const int sb_off = (lane & 31) * 16;
+  const bool sb_lane = sb_off < quad_sb_bytes;
+  // where this lane finds the scale of piece (j, blk) of row li inside a region
+  const int piece_groups = (16 * kCodes) >> gs_shift;  // groups one load instruction spans
+  const int sidx0 = (li * groups + ((blk * kCodes) >> gs_shift)) * 2;
+
+  uint32_t pair_mask = (BITS == 8 && CF::kWholeByte) ? 0x00ff00ffu : 0x000f000fu;
+  uint32_t magic = CF::kNibble, magic_high = CF::kHighMagic;
+  asm volatile("" : "+s"(pair_mask), "+v"(magic), "+v"(magic_high));
+
+  auto load_scales = [&](int q) __attribute__((always_inline)) {
+    u32x4 v = {0, 0, 0, 0};
+    if (sb_lane) v = *reinterpret_cast<const u32x4*>(sb_src + (size_t)q * quad_sb_bytes + sb_off);
+    return v;
+  };
+  auto store_scales = [&](u32x4 v, int buf) __attribute__((always_inline)) {
+    *reinterpret_cast<u32x4*>(sreg + buf * kScaleRegion + (lane >> 5) * 512 + sb_off) = v;
+  };
+  auto load_piece = [&](int q, int j) __attribute__((always_inline)) {
+    return __builtin_nontemporal_load(
+        reinterpret_cast<const u32x4*>(wbytes + (size_t)q * 4 * row_bytes + lane_woff + 256 * j));
+  };
+
+  // The first weight pieces and the first quad's scales are requested before
+  // anything else, so that their latency overlaps the staging of x.
+  u32x4 ring[kRing];
+  const int q_first = has_work ? q_begin : 0;
+#pragma unroll
+  for (int j = 0; j < kRing; ++j) ring[j] = load_piece(q_first, j);
+  const u32x4 sb_first = load_scales(q_first);
+
+  // ---- x: the B operands and the slice sums of every lane position, computed
+  // once per workgroup (the four wavefronts share the pieces out) and kept in
+  // LDS; every wavefront then reads back the sums of its own lanes
+  for (int j = wave; j < kLoads; j += 4) {
+    const int k0 = (j * 16 + blk) * kCodes;
+    float sum = 0.f;
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) {  // the piece's four words
+      if constexpr (BITS == 4) {
+        // word = codes c0..c7; pairs (c0,c4) (c1,c5) | (c2,c6) (c3,c7)
+        u32x4 v = {0, 0, 0, 0};
+        if (li < M) v = *reinterpret_cast<const u32x4*>(x + (int64_t)li * K + k0 + 8 * wd);
+        *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd) * 64 + lane) * 8) =
+            make_uint2((v[0] & 0xffffu) | (v[2] << 16), (v[0] >> 16) | (v[2] & 0xffff0000u));
+        *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd + 1) * 64 + lane) * 8) =
+            make_uint2((v[1] & 0xffffu) | (v[3] << 16), (v[1] >> 16) | (v[3] & 0xffff0000u));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum += T::to_f32((uint16_t)v[e]) + T::to_f32((uint16_t)(v[e] >> 16));
+      } else {
+        // word = codes c0..c3; pairs (c0,c2) (c1,c3)
+        uint2 v = {0, 0};
+        if (li < M) v = *reinterpret_cast<const uint2*>(x + (int64_t)li * K + k0 + 4 * wd);
+        *reinterpret_cast<uint2*>(lds + ((j * kXOps + wd) * 64 + lane) * 8) =
+            make_uint2((v.x & 0xffffu) | (v.y << 16), (v.x >> 16) | (v.y & 0xffff0000u));
+        sum += T::to_f32((uint16_t)v.x) + T::to_f32((uint16_t)(v.x >> 16)) + T::to_f32((uint16_t)v.y) +
+               T::to_f32((uint16_t)(v.y >> 16));
+      }
+    }
+    *reinterpret_cast<float*>(lds + kXBytes + (j * 64 + lane) * 4) = sum;
+  }
+  __syncthreads();
+  float sx[kLoads];
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) sx[j] = *reinterpret_cast<const float*>(lds + kXBytes + (j * 64 + lane) * 4);
+  const char* xops = lds + lane * 8;
+
+  if (!has_work) return;
+  store_scales(sb_first, q_begin & 1);
+
+  for (int q = q_begin; q < q_end; ++q) {
+    const int qn = min(q + 1, q_end - 1);  // past the end: this wavefront's last quad again, never consumed
+    const u32x4 sb_next = load_scales(qn);
+    const char* sb = sreg + (q & 1) * kScaleRegion + sidx0;
+    f32x4 tot = {0.f, 0.f, 0.f, 0.f};  // register i: row r0+i against this lane's activation row
+    for_each_index<kLoads>([&](auto jc) __attribute__((always_inline)) {
+      constexpr int j = decltype(jc)::value;
+      constexpr int slot = j % kRing;
+      const float sc = T::to_f32(*reinterpret_cast<const uint16_t*>(sb + j * piece_groups * 2));
+      const float bi = T::to_f32(*reinterpret_cast<const uint16_t*>(sb + 512 + j * piece_groups * 2));
+      const float bo = __builtin_fmaf(-kOffset, sc, bi);
+      // two accumulation chains, so that a matrix instruction need not wait for the one before it
+      f32x4 d = {0.f, 0.f, 0.f, 0.f}, d2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd) {
+        const uint32_t w = ring[slot][wd];
+        if constexpr (BITS == 4) {
+          const uint2 a0 = make_uint2((w & pair_mask) | magic, ((w >> 4) & pair_mask) | magic);
+          const uint2 a1 = make_uint2(((w >> 8) & pair_mask) | magic, ((w >> 12) & pair_mask) | magic);
+          d = CF::mfma4(a0, *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd) * 512), d);
+          d2 = CF::mfma4(a1, *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd + 1) * 512), d2);
+        } else if constexpr (CF::kWholeByte) {
+          const uint2 a = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
+          const uint2 xb = *reinterpret_cast<const uint2*>(xops + (j * kXOps + wd) * 512);
+          if (wd & 1) {
+            d2 = CF::mfma4(a, xb, d2);
+          } else {
+            d = CF::mfma4(a, xb, d);
+          }
+        } else {
+          const uint2 lo = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
+          const uint2 hi = make_uint2(((w >> 4) & pair_mask) | magic_high, ((w >> 12) & pair_mask) | magic_high);
+          const uint2 xb = *reinterpret_cast<const uint2*>(xops + (j * kXOps + wd) * 512);
+          d = CF::mfma4(lo, xb, d);
+          d2 = CF::mfma4(hi, xb, d2);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) d[e] += d2[e];
+      // refill the slot: the piece kRing further on, in this quad or the next
+      if constexpr (j + kRing < kLoads) {
+        ring[slot] = load_piece(q, j + kRing);
+      } else {
+        ring[slot] = load_piece(qn, j + kRing - kLoads);
+      }
+      // keep the refills in place (left to itself the scheduler sinks the loads
+      // behind several pieces of arithmetic and the ring runs dry), but let the
+      // arithmetic of two pieces interleave
+      if constexpr (j % 2 == 1 || j == kLoads - 1) __builtin_amdgcn_sched_barrier(0);
+      // register i belongs to row r0+i, whose scale and bias lane i of the quad holds
+      tot[0] = __builtin_fmaf(dpp_f32<0x00>(sc), d[0], tot[0]);
+      tot[1] = __builtin_fmaf(dpp_f32<0x55>(sc), d[1], tot[1]);
+      tot[2] = __builtin_fmaf(dpp_f32<0xAA>(sc), d[2], tot[2]);
+      tot[3] = __builtin_fmaf(dpp_f32<0xFF>(sc), d[3], tot[3]);
+      tot[0] = __builtin_fmaf(dpp_f32<0x00>(bo), sx[j], tot[0]);
+      tot[1] = __builtin_fmaf(dpp_f32<0x55>(bo), sx[j], tot[1]);
+      tot[2] = __builtin_fmaf(dpp_f32<0xAA>(bo), sx[j], tot[2]);
+      tot[3] = __builtin_fmaf(dpp_f32<0xFF>(bo), sx[j], tot[3]);
+    });
+    // the other region was last read one quad ago
+    store_scales(sb_next, (q + 1) & 1);
+
+    // add up the 16 blocks: lanes with the same lane%4
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = tot[i];
+      v += dpp_f32<kDppRowRor4>(v);
+      v += dpp_f32<kDppRowRor8>(v);
+      v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) * 4, __builtin_bit_cast(int, v)));
+      v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, __builtin_bit_cast(int, v)));
+      tot[i] = v;
+    }
+    if (lane < M) {  // lane m holds y[m, r0..r0+3]
+      const int64_t r0 = (int64_t)q * 4;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[i] = T::to_f32(bias[r0 + i]);
+      }
+      const int64_t o = (int64_t)lane * N + r0;
+      if (y_is_f32) {
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(y) + o) =
+            make_float4(tot[0] + bv[0], tot[1] + bv[1], tot[2] + bv[2], tot[3] + bv[3]);
+      } else {
+        uint32_t pk[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          pk[c] = T::pack2(tot[2 * c], tot[2 * c + 1]);
+          if (bias)  // second rounding, as a separate add on the 16-bit result would do
+            pk[c] = T::pack2(T::to_f32((uint16_t)pk[c]) + bv[2 * c], T::to_f32((uint16_t)(pk[c] >> 16)) + bv[2 * c + 1]);
+        }
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(y) + o) = make_uint2(pk[0], pk[1]);
+      }
+    }
+  }
+}
+
+template <typename T, int BITS, int kLoads, int kRing>
+int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                  const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
+  auto kernel = qmv_quad_kernel<T, BITS, kLoads, kRing>;
+  constexpr int kXOps = 128 / BITS / 4;
+  constexpr int kLds = kLoads * kXOps * 512 + kLoads * 256 + 4 * 2 * kScaleRegion;
+  static int blocks_per_cu = 0;
+  if (blocks_per_cu == 0) {
+    if (kLds > 48 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) !=
+            hipSuccess)
+      return MFQ_ELAUNCH;
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, kLds) != hipSuccess || n < 1) n = 1;
+    blocks_per_cu = n > 4 ? 4 : n;
+  }
+  // At most as many wavefronts as are resident at once, and every one of them
+  // the same number of quads: with 4608 quads, 2304 wavefronts of two finish
+  // together, whereas 4096 wavefronts would leave 512 of them a second quad.
+  const int64_t quads = N / 4;
+  const int64_t max_waves = (int64_t)compute_units() * blocks_per_cu * 4;
+  const int64_t per_wave = (quads + max_waves - 1) / max_waves;
+  const int64_t n_waves = (quads + per_wave - 1) / per_wave;
+  const int64_t blocks = (n_waves + 3) / 4;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), kLds, stream, (const uint16_t*)x, wq,
+                     (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, gs_shift, (int)per_wave);
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T, int BITS>
+int launch_loads(int64_t loads, const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                 const void* biases, const void* bias, int64_t N, int gs_shift, void* y, int y_dtype,
+                 hipStream_t stream) {
+#define MFQ_QUAD_CASE(L, R)                                                                                      \
+  case L:                                                                                                        \
+    return launch_kernel<T, BITS, L, R>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream)
+  switch (loads) {
+    MFQ_QUAD_CASE(1, 1);
+    MFQ_QUAD_CASE(2, 2);
+    MFQ_QUAD_CASE(3, 3);
+    MFQ_QUAD_CASE(4, 4);
+    MFQ_QUAD_CASE(6, 6);
+    MFQ_QUAD_CASE(8, 4);
+    MFQ_QUAD_CASE(12, 6);
+    MFQ_QUAD_CASE(16, 4);
+    default:
+      return MFQ_EUNSUPPORTED;
+  }
+#undef MFQ_QUAD_CASE
+}
+
+}  // namespace
+
+// Shapes this kernel takes: M <= 4; whole quads of rows; rows that are a
+// supported number of 256-byte pieces; at most 64 groups per row, an even
+// number (the staged scale block of a quad is 16-byte pieces of at most 512
+// bytes); K <= 4096 (the x operands' LDS copy); pointers aligned for the
+// 16-byte scale fetches and the 8- / 16-byte stores.
+bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* scales, const void* biases,
+                     const void* y, int y_dtype) {
+  const int64_t row_bytes = K * bits / 8;
+  const int64_t loads = row_bytes / 256;
+  const int64_t groups = K / gs;
+  const bool loads_ok = row_bytes % 256 == 0 && (loads == 1 || loads == 2 || loads == 3 || loads == 4 || loads == 6 ||
+                                                 loads == 8 || loads == 12 || loads == 16);
+  const uintptr_t y_mask = y_dtype == MFQ_F32 ? 15u : 7u;
+  return M >= 1 && M <= 4 && N % 4 == 0 && loads_ok && groups <= 64 && groups % 2 == 0 && K <= 4096 &&
+         aligned16(scales) && aligned16(biases) && (reinterpret_cast<uintptr_t>(y) & y_mask) == 0;
+}
+
+int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                    hipStream_t stream) {
+  const int gs_shift = gs == 32 ? 5 : gs == 64 ? 6 : 7;
+  const int64_t loads = K * bits / 8 / 256;
+  if (dtype == MFQ_BF16) {
+    if (bits == 4)
+      return launch_loads<BF16, 4>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    return launch_loads<BF16, 8>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+  }
+  if (dtype == MFQ_F16) {
+    if (bits == 4)
+      return launch_loads<F16, 4>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    return launch_loads<F16, 8>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+  }
+  return MFQ_EDTYPE;
+}
+
+}  // namespace mfq

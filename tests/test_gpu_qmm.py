@@ -94,6 +94,57 @@ def test_qmv_few_rows_short_k(oracle, bits, M):
         _assert_close(_run(o, *args, bits), _ref(o, *args, bits))
 
 
+@pytest.mark.parametrize("bits,gs,K", [
+    (8, 64, 256), (8, 64, 512), (8, 64, 768), (8, 64, 1024), (8, 64, 1536), (8, 64, 2048), (8, 64, 3072), (8, 64, 4096),
+    (4, 64, 512), (4, 64, 1024), (4, 64, 1536), (4, 64, 2048), (4, 64, 3072), (4, 64, 4096),
+    (8, 128, 3072), (4, 128, 4096), (8, 32, 1024), (4, 32, 2048), (8, 32, 256),
+])
+@pytest.mark.parametrize("M", [2, 4])
+def test_qmv_four_rows_at_a_time(oracle, bits, gs, K, M):
+    """M = 2..4 through the kernel that takes four weight rows at a time: every
+    number of 256-byte pieces per row it is built for, all group sizes, runs of
+    quads of uneven length, bf16 with bias and float32 output."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    N = 4 * 1031 if K <= 1024 else 4 * 53
+    args = _case(o, 41, M, K, N, bits, gs=gs)
+    ref = _ref(o, *args, bits, gs)
+    _assert_close(_run(o, *args, bits, gs), ref)
+    x, wq, s, b, bias = args
+    y32 = mflux_amd.quantized_matmul(to_dev(x, o.BF16).float(), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                     group_size=gs, bits=bits, bias=to_dev(bias, o.BF16))
+    assert y32.dtype == torch.float32
+    _assert_close(y32, ref, tol=2e-3)  # nothing is rounded to 16 bits on this path
+
+
+def test_qmv_four_rows_one_hot(oracle):
+    """One-hot activation rows (a different k in each of the four rows) return
+    four columns of the weight: every (piece, block, word) position of the
+    four-rows-at-a-time kernel against scale * code + bias."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    K, N = 3072, 64
+    w = o.f32_to_bf16_bits(seeded(42, 1, (N, K), 0.02))
+    for bits in (4, 8):
+        wq, s, b = o.c_quantize(w, o.BF16, 64, bits)
+        exact = o.dequantize_exact(wq, s, b, o.BF16, 64, bits).astype(np.float64)
+        step = np.abs(o.bf16_bits_to_f32(s).astype(np.float64))
+        for k0 in (0, 5, 16, 33, 255, 256, 1000, 2047, 3068):
+            ks = [k0, (k0 + 1) % K, (k0 + 17) % K, (k0 + 1531) % K]
+            xf = np.zeros((4, K), dtype=np.float32)
+            for m, k in enumerate(ks):
+                xf[m, k] = 1.0
+            y = mflux_amd.quantized_matmul(to_dev(o.f32_to_bf16_bits(xf), o.BF16).float(), u32_to_dev(wq),
+                                           to_dev(s, o.BF16), to_dev(b, o.BF16), group_size=64, bits=bits)
+            got = y.cpu().numpy().astype(np.float64)
+            for m, k in enumerate(ks):
+                assert np.all(np.abs(got[m] - exact[:, k]) <= 1e-3 * step[:, k // 64]), (bits, k0, m)
+
+
 def test_qmv_one_hot_and_float32_output(oracle):
     """One-hot x through the one-row kernel returns a column of the weight, for
     every lane position of every load.  The kernel multiplies x with the raw
