@@ -133,11 +133,12 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
 
 /*
  * mfq_qmm_t with an optional float32 workspace.  Has no counterpart in the
- * reference (MLX allocates inside its ops).  Shapes with fewer output tiles
- * than the GPU has compute units -- the text-stream linears of the double
+ * reference (MLX allocates inside its ops).  Shapes whose output tiles do not
+ * fill the GPU's compute units -- the text-stream linears of the double
  * blocks, M = 256 or 512 tokens against N = 3072, e.g.
  * src/mflux/models/qwen/model/qwen_transformer/qwen_transformer_block.py:36-37
- * on the caption tokens -- leave part of the chip idle; with a workspace K is
+ * on the caption tokens, or the last, mostly empty round of tiles of the image
+ * stream at M = 6889 -- leave part of the chip idle; with a workspace K is
  * cut into ranges that run on different compute units, each range accumulates
  * into its own float32 plane of the workspace, and a second kernel adds the
  * planes, rounds and applies the bias (same two roundings as the fused

@@ -128,49 +128,76 @@ struct ScaleRegs {
   }
 };
 
+// Position `tile` of the tile sequence -> origin of the tile.  Workgroups are
+// dealt round-robin to the 8 XCDs, so with a grid that is a multiple of 8 a
+// workgroup stays on XCD b%8 and that XCD's workgroups walk a contiguous run of
+// the sequence together.  Inside the run the tiles are ordered in bands of
+// kBandM tile-rows, row index fastest, so the ~32 tiles in flight on one XCD
+// share kBandM x-tiles and 8 weight-tiles per k step in that XCD's L2.
+__host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, int& m0, int& n0) {
+  const int n_tiles = tiles_m * tiles_n;
+  const int per_xcd = n_tiles / 8;
+  if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
+  constexpr int kBandM = 4;
+  const int band_tiles = kBandM * tiles_n;
+  const int band = tile / band_tiles;
+  const int rest = tiles_m - band * kBandM;
+  const int band_rows = rest < kBandM ? rest : kBandM;
+  const int in_band = tile - band * band_tiles;
+  m0 = (band * kBandM + in_band % band_rows) * BM;
+  n0 = (in_band / band_rows) * BN;
+}
+
 template <typename T, int GS, int BITS, bool kFast>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
-    int N, int K, int tiles_m, int tiles_n, int splits, int steps) {
+    int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits, float* __restrict__ planes) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   using WR = WeightRegs<T, GS, BITS>;
   using SR = ScaleRegs<T, GS>;
 
   const int n_tiles = tiles_m * tiles_n;
-  const int n_items = n_tiles * splits;  // work items: (tile, k range); splits == 1 unless the launcher split K
+  // work items: the first n_whole tiles of the sequence whole, every later tile as tail_splits k ranges
+  const int n_items = n_whole + (n_tiles - n_whole) * tail_splits;
+  const int steps_total = K / BK;
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
   const int wn = wave * 64;
   const int r = lane & 31;
   const int h = lane >> 5;
-  // `steps`: k steps of one work item (K / BK when K is not split)
 
   // Persistent workgroups: workgroup b takes items b, b + grid, b + 2*grid, ...
-  // Item i is k range i / n_tiles of tile i % n_tiles: with K split, range s of
-  // every tile goes to float32 plane s of the workspace `y` points at, and a
-  // second kernel adds the planes up.
-  // Workgroups are dealt round-robin to the 8 XCDs, so with a grid that is a
-  // multiple of 8 a workgroup stays on XCD b%8 and that XCD's workgroups walk
-  // a contiguous run of the tile sequence together.  Inside the run the tiles
-  // are ordered in bands of kBandM tile-rows, row index fastest, so the ~32
-  // tiles in flight on one XCD share kBandM x-tiles and 8 weight-tiles per k
-  // step in that XCD's L2.
-  auto tile_origin = [&](int seq, int& m0, int& n0, int& split) {
-    split = seq / n_tiles;
-    int tile = seq - split * n_tiles;
-    const int per_xcd = n_tiles / 8;
-    if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
-    constexpr int kBandM = 4;
-    const int band_tiles = kBandM * tiles_n;
-    const int band = tile / band_tiles;
-    const int band_rows = min(tiles_m - band * kBandM, kBandM);
-    const int in_band = tile - band * band_tiles;
-    m0 = (band * kBandM + in_band % band_rows) * BM;
-    n0 = (in_band / band_rows) * BN;
+  // The launcher makes the whole tiles a whole number of rounds; what is left
+  // of the tile sequence (fewer tiles than compute units) can be cut along K
+  // so that the last round is short instead of mostly idle: k range s of tail
+  // tile t accumulates into float32 plane t * tail_splits + s (256 x 256,
+  // dense) of `planes`, and a second kernel adds the planes into y.
+  struct Item {
+    int m0, n0;
+    int first_step, n_steps;  // its k range, in steps
+    int plane;                // -1: the whole tile, written to y; else the index of its float32 plane
   };
+  auto item_of = [&](int seq) {
+    Item it;
+    int tile = seq;
+    it.first_step = 0;
+    it.n_steps = steps_total;
+    it.plane = -1;
+    if (seq >= n_whole) {
+      const int e = seq - n_whole;
+      const int tail_tile = e / tail_splits;
+      tile = n_whole + tail_tile;
+      it.n_steps = steps_total / tail_splits;
+      it.first_step = (e - tail_tile * tail_splits) * it.n_steps;
+      it.plane = e;
+    }
+    tile_origin(tile, tiles_m, tiles_n, it.m0, it.n0);
+    return it;
+  };
+  int steps = steps_total;  // k steps of the item in hand
 
   // Per-lane byte offsets of the tile the PREFETCH cursor is in (it runs two k
   // steps ahead of the matrix work and enters the next tile two steps early;
@@ -208,7 +235,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // x tile registers: set p receives the tile of a step with parity p, two
   // steps before it is used, and is published to LDS buffer p one step before.
   u32x4 xa[2][8];
-  char* y_item = static_cast<char*>(y);  // where the current item's results go
+  // where the item in hand writes its results: the address of element (m0, n0),
+  // the row pitch in elements, the element type and the bias to add (planes:
+  // float32, 256 apart, no bias)
+  char* out_base = static_cast<char*>(y);
+  int out_stride = N;
+  bool out_f32 = y_is_f32;
+  const uint16_t* out_bias = bias;
   WR wa, wb;            // packed weights of the current even / odd step
   SR sr;                // scales and biases of the period the prefetch cursor is in (kFast only)
   uint32_t bf[2][4];    // dequantised fragments of the next sub-step to run
@@ -398,16 +431,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     asm volatile("" : "+v"(lane_e));
     const int r = lane_e & 31;
     const int h = lane_e >> 5;
-    const bool n_vec_ok = (N & 3) == 0;  // keeps every piece aligned and inside the row
+    const bool n_vec_ok = (N & 3) == 0 && (out_stride & 3) == 0;  // keeps every piece aligned and inside the row
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int eb = 0; eb < 4; ++eb) {
         const int col = n0 + wn + 32 * j + 8 * eb + 4 * h;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias) {
+        if (out_bias) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(col + c, N - 1)]);
+          for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(out_bias[min(col + c, N - 1)]);
         }
 #pragma unroll
         for (int ai = 0; ai < 8; ++ai) {
@@ -416,10 +449,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           float v[4];
 #pragma unroll
           for (int c = 0; c < 4; ++c) v[c] = acc[ai][j][4 * eb + c];
-          const int64_t o = (int64_t)row * N + col;
-          if (y_is_f32) {
-            float* dst = reinterpret_cast<float*>(y_item) + o;
-            if (bias) {
+          const int64_t o = (int64_t)(row - m0) * out_stride + (col - n0);
+          if (out_f32) {
+            float* dst = reinterpret_cast<float*>(out_base) + o;
+            if (out_bias) {
 #pragma unroll
               for (int c = 0; c < 4; ++c) v[c] += bv[c];
             }
@@ -435,9 +468,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
               hv[c] = T::from_f32(v[c]);
-              if (bias) hv[c] = T::from_f32(T::to_f32(hv[c]) + bv[c]);
+              if (out_bias) hv[c] = T::from_f32(T::to_f32(hv[c]) + bv[c]);
             }
-            uint16_t* dst = reinterpret_cast<uint16_t*>(y_item) + o;
+            uint16_t* dst = reinterpret_cast<uint16_t*>(out_base) + o;
             if (n_vec_ok) {
               uint2 pk;
               pk.x = (uint32_t)hv[0] | ((uint32_t)hv[1] << 16);
@@ -472,7 +505,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int h = lane_e >> 5;
     const int lane = lane_e;
     char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
-    uint16_t* yout = reinterpret_cast<uint16_t*>(y_item);
+    uint16_t* yout = reinterpret_cast<uint16_t*>(out_base);
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
@@ -483,7 +516,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           float bv[4] = {0.f, 0.f, 0.f, 0.f};
           if constexpr (kBias) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(n0 + wn + cl + c, N - 1)]);
+            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(out_bias[min(n0 + wn + cl + c, N - 1)]);
           }
 #pragma unroll
           for (int a4 = 0; a4 < 4; ++a4) {
@@ -508,7 +541,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int rl = 8 * k + (lane >> 3);
         const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
         const int row = m0 + 128 * pass + rl;
-        if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
+        if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
         if (k & 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -527,7 +560,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int h = lane_e >> 5;
     const int lane = lane_e;
     char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
-    float* yout = reinterpret_cast<float*>(y_item);
+    float* yout = reinterpret_cast<float*>(out_base);
 #pragma unroll
     for (int pass = 0; pass < 4; ++pass) {
 #pragma unroll
@@ -536,9 +569,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         for (int eb = 0; eb < 4; ++eb) {
           const int cl = 32 * j + 8 * eb + 4 * h;  // column inside the wavefront's 64
           float bv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (bias) {
+          if (out_bias) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(n0 + wn + cl + c, N - 1)]);
+            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(out_bias[min(n0 + wn + cl + c, N - 1)]);
           }
 #pragma unroll
           for (int a2 = 0; a2 < 2; ++a2) {
@@ -557,19 +590,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int rl = 4 * k + (lane >> 4);
         const float4 v = *reinterpret_cast<const float4*>(stage + rl * kStride + 16 * (lane & 15));
         const int row = m0 + 64 * pass + rl;
-        if (row < M && cg < N) *reinterpret_cast<float4*>(yout + (int64_t)row * N + cg) = v;
+        if (row < M && cg < N) *reinterpret_cast<float4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
         if (k & 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
   auto store_tile = [&](int m0, int n0) {
-    if (!y_is_f32 && (N & 7) == 0) {
-      if (bias) {
+    if (!out_f32 && (out_stride & 7) == 0 && (N & 7) == 0) {
+      if (out_bias) {
         store_tile_staged(std::true_type{}, m0, n0);
       } else {
         store_tile_staged(std::false_type{}, m0, n0);
       }
-    } else if (y_is_f32 && (N & 3) == 0) {
+    } else if (out_f32 && (out_stride & 3) == 0 && (N & 3) == 0) {
       store_tile_staged_f32(m0, n0);
     } else {
       store_tile_direct(m0, n0);
@@ -578,12 +611,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   bool primed = false;
   for (int seq = blockIdx.x; seq < n_items; seq += gridDim.x) {
-    int m0, n0, split;
-    tile_origin(seq, m0, n0, split);
-    const int kb = split * steps * BK;            // first k of this item
+    const Item item = item_of(seq);
+    const int m0 = item.m0, n0 = item.n0;
+    steps = item.n_steps;
+    const int kb = item.first_step * BK;          // first k of this item
     constexpr int kGroupsPerStep2 = 2 * BK / GS;  // groups per step, times two (GS == 128: one)
-    const int gb = split * steps * kGroupsPerStep2 / 2;  // its first group
-    y_item = static_cast<char*>(y) + (size_t)split * M * N * 4;  // split > 0 only with float32 planes
+    const int gb = item.first_step * kGroupsPerStep2 / 2;  // its first group
+    if (item.plane < 0) {
+      out_base = static_cast<char*>(y) + ((size_t)m0 * N + n0) * (y_is_f32 ? 4 : 2);
+      out_stride = N;
+      out_f32 = y_is_f32;
+      out_bias = bias;
+    } else {
+      out_base = reinterpret_cast<char*>(planes + (size_t)item.plane * (BM * BN));
+      out_stride = BN;
+      out_f32 = true;
+      out_bias = nullptr;
+    }
     if (!primed) {
       set_scale_tile(n0);
       set_prefetch_tile(m0, n0);
@@ -629,9 +673,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
       {
         const int p = steps - kPer;  // first step of the last period
-        int m1 = m0, n1 = n0, split1 = split;
-        if (has_next) tile_origin(seq + gridDim.x, m1, n1, split1);
-        const int kb1 = split1 * steps * BK, gb1 = split1 * steps * kGroupsPerStep2 / 2;  // the next item's first k, group
+        Item next = item;
+        if (has_next) next = item_of(seq + gridDim.x);
+        const int m1 = next.m0, n1 = next.n0;
+        const int kb1 = next.first_step * BK, gb1 = next.first_step * kGroupsPerStep2 / 2;  // the next item's first k, group
         const int g_last = gb + p * kGroupsPerStep2 / 2;  // this item's last period, for prefetches nobody consumes
         const int k_last = kb + (steps - 2) * BK;
         if constexpr (kPer >= 4) {
@@ -651,7 +696,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       primed = has_next;
     } else {
       int step = 0;
-      for (; step + 1 < steps; step += 2) {  // never split: kb == 0
+      for (; step + 1 < steps; step += 2) {  // never cut along K: kb == 0
         do_step(even_step, keep, wa, wb, min(step + 2, steps - 1) * BK, 0, 0);
         do_step(odd_step, keep, wb, wa, min(step + 3, steps - 1) * BK, 0, 0);
       }
@@ -667,26 +712,35 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 }
 
-// ---- K split across workgroups (few tiles, long K) -------------------------
-// With fewer than half as many 256 x 256 tiles as there are CUs, K is cut into
-// `splits` equal ranges of whole periods; range s of every tile is accumulated
-// into float32 plane s of a caller-provided workspace and the planes are added
-// up, rounded and biased by splitk_reduce_kernel.
-struct SplitPlan {
-  int splits;
-  int steps;  // k steps per range
+// ---- the last round of tiles cut along K ---------------------------------------
+// The tiles that fill whole rounds of the compute units run whole.  The tail of
+// the sequence -- fewer tiles than compute units, which would keep most of the
+// chip idle for a full tile time -- is cut into `splits` equal k ranges of whole
+// scale periods when a caller-provided workspace is there: every range goes to
+// its own dense 256 x 256 float32 plane and tail_reduce_kernel adds the planes
+// up, rounds and applies the bias.
+struct TailPlan {
+  int n_whole;  // tiles of the sequence that run whole
+  int splits;   // k ranges per tail tile; 1: nothing is cut
 };
 
-// period: k steps per scale period of the group size.  The largest number of
-// equal ranges of whole periods (at least 4 steps each) that keeps one work
-// item per CU.
-inline SplitPlan plan_split(int64_t M, int64_t N, int64_t K, int period, int cus) {
+// period: k steps per scale period of the group size.  The cut must pay for
+// its planes: a range saves steps - steps/splits k steps of about 1.6 us each
+// on the critical path, a plane costs about 0.13 us of memory traffic (256 KiB
+// written and read back) plus the second launch.
+inline TailPlan plan_tail(int64_t M, int64_t N, int64_t K, int period, int cus) {
   const int steps = (int)(K / BK);
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  SplitPlan plan{1, steps};
-  if (steps % period != 0 || steps < 4 || tiles * 2 > cus) return plan;
-  for (int s = 2; s <= steps / 4 && tiles * s <= cus; ++s)
-    if (steps % s == 0 && (steps / s) % period == 0) plan = SplitPlan{s, steps / s};
+  const int64_t tail = tiles % cus;
+  TailPlan plan{(int)tiles, 1};
+  if (tail == 0 || steps % period != 0 || steps < 8) return plan;
+  int best = 1;
+  for (int s = 2; s <= steps / 4 && tail * s <= cus; ++s)
+    if (steps % s == 0 && (steps / s) % period == 0) best = s;
+  if (best == 1) return plan;
+  const double saved_us = 1.6 * (steps - steps / best);
+  const double cost_us = 0.13 * (double)tail * best + 6.0;
+  if (saved_us > 1.25 * cost_us) plan = TailPlan{(int)(tiles - tail), best};
   return plan;
 }
 
@@ -741,9 +795,44 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
+// y tile = sum of the `splits` planes of each tail tile (+ bias).  One thread per
+// four consecutive columns of a tile row.
+template <typename T>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restrict__ planes, int n_whole, int splits,
+                                                          int tiles_m, int tiles_n, const uint16_t* __restrict__ bias,
+                                                          int M, int N, void* __restrict__ y, int y_is_f32) {
+  const int tail_tile = blockIdx.x / (BM * BN / 4 / 256);
+  const int q = (blockIdx.x % (BM * BN / 4 / 256)) * 256 + threadIdx.x;  // quad inside the tile
+  const int r = q / (BN / 4), c = (q % (BN / 4)) * 4;
+  int m0, n0;
+  tile_origin(n_whole + tail_tile, tiles_m, tiles_n, m0, n0);
+  const int row = m0 + r, col = n0 + c;
+  if (row >= M || col >= N) return;
+  const float* src = planes + (size_t)tail_tile * splits * (BM * BN) + r * BN + c;
+  float4 sum = *reinterpret_cast<const float4*>(src);
+  for (int sp = 1; sp < splits; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * (BM * BN));
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  }
+  float v[4] = {sum.x, sum.y, sum.z, sum.w};
+  const int64_t o = (int64_t)row * N + col;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (col + e >= N) break;
+    const float bv = bias ? T::to_f32(bias[col + e]) : 0.f;
+    if (y_is_f32) {
+      reinterpret_cast<float*>(y)[o + e] = v[e] + bv;
+    } else {  // round, then add the bias and round again, as the fused epilogue does
+      uint16_t hv = T::from_f32(v[e]);
+      if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
+      reinterpret_cast<uint16_t*>(y)[o + e] = hv;
+    }
+  }
+}
+
 template <typename T, int GS, int BITS, bool kFast>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                  const void* bias, int64_t N, void* y, int y_dtype, SplitPlan plan, hipStream_t stream) {
+                  const void* bias, int64_t N, void* y, int y_dtype, TailPlan plan, void* planes, hipStream_t stream) {
   auto kernel = qmm_kernel<T, GS, BITS, kFast>;
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
   if (!configured) {
@@ -754,12 +843,27 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   }
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
-  const int n_items = tiles_m * tiles_n * plan.splits;
+  const int n_tail = tiles_m * tiles_n - plan.n_whole;
+  const int n_items = plan.n_whole + n_tail * plan.splits;
   const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
-                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.splits, plan.steps);
-  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.n_whole, plan.splits,
+                     (float*)planes);
+  if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
+  if (plan.splits > 1) {
+    const unsigned blocks = (unsigned)n_tail * (BM * BN / 4 / 256);
+    hipLaunchKernelGGL((tail_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, (const float*)planes, plan.n_whole,
+                       plan.splits, tiles_m, tiles_n, (const uint16_t*)bias, (int)M, (int)N, y,
+                       (int)(y_dtype == MFQ_F32));
+    if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
+  }
+  return MFQ_OK;
+}
+
+inline size_t tail_plane_bytes(int64_t M, int64_t N, TailPlan plan) {
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  return plan.splits > 1 ? (size_t)(tiles - plan.n_whole) * plan.splits * BM * BN * sizeof(float) : 0;
 }
 
 template <typename T, int GS, int BITS>
@@ -768,23 +872,19 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
                hipStream_t stream) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const TailPlan whole{(int)tiles, 1};
   // period-wise scale loads: whole periods, at least two pairs of steps, and
   // 8-byte aligned scale rows
   const int64_t steps = K / BK;
   constexpr int kPer = ScaleRegs<T, GS>::kPeriod;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
   if (!(steps % kPer == 0 && steps >= 4 && aligned8))
-    return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype,
-                                             SplitPlan{1, (int)steps}, stream);
-  const SplitPlan plan = plan_split(M, N, K, kPer, compute_units());
-  const size_t need = (size_t)plan.splits * M * N * sizeof(float);
-  if (plan.splits == 1 || !workspace || workspace_bytes < need || !aligned16(workspace))
-    return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype,
-                                            SplitPlan{1, (int)steps}, stream);
-  if (int rc = launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
-                                                stream))
-    return rc;
-  return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
+    return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, whole, nullptr, stream);
+  TailPlan plan = plan_tail(M, N, K, kPer, compute_units());
+  if (plan.splits > 1 && (!workspace || workspace_bytes < tail_plane_bytes(M, N, plan) || !aligned16(workspace)))
+    plan = whole;
+  return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, workspace, stream);
 }
 
 template <typename T, int GS>
@@ -819,8 +919,7 @@ inline bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
   if (K % BK) return 0;
   if (use_mid_kernel(M, N, K)) return qmm_mid_workspace_bytes(M, N, K, gs);
-  const SplitPlan plan = plan_split(M, N, K, period_of(gs), compute_units());
-  return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+  return tail_plane_bytes(M, N, plan_tail(M, N, K, period_of(gs), compute_units()));
 }
 
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,

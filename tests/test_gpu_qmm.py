@@ -217,6 +217,29 @@ def test_qmm_split_k_shapes(oracle, bits, gs, M, K, N):
     _assert_close(y32, ref, tol=5e-3)  # float32 output: only the weights' 16-bit rounding remains
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qmm_last_round_cut_along_k(oracle, bits):
+    """270 tiles on a 256-CU GPU: the first 256 run whole, the 14 of the last
+    round are cut along K into float32 planes that a second kernel adds up
+    (ragged M and N, bias; bf16 and float32 output)."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    M, K, N = 2200, 2048, 7504
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert _lib.load().mfq_qmm_t_workspace_bytes(M, K, N, 64, bits) == 14 * 8 * 256 * 256 * 4
+    args = _case(o, 34, M, K, N, bits)
+    ref = _ref(o, *args, bits)
+    _assert_close(_run(o, *args, bits), ref)
+    x, wq, s, b, bias = args
+    y32 = mflux_amd.quantized_matmul(to_dev(x, o.BF16).float(), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                     group_size=64, bits=bits, bias=to_dev(bias, o.BF16))
+    assert y32.dtype == torch.float32
+    _assert_close(y32, ref, tol=5e-3)
+
+
 def test_qmm_split_k_matches_unsplit_through_c_abi(oracle):
     """mfq_qmm_t (no workspace) and mfq_qmm_t_ws (split) on the same operands:
     both within tolerance of the oracle and of each other; a too-small
@@ -447,7 +470,7 @@ def test_qmm_medium_m_odd_n(oracle):
 @pytest.mark.parametrize("bits,gs", [(4, 64), (8, 128)])
 def test_qmm_many_rows_long_k_split(oracle, bits, gs):
     """More than 512 rows, few 256 x 256 tiles and K >= 8192: the large-M
-    kernel with K cut across compute units."""
+    kernel with every tile cut along K across compute units."""
     from mflux_amd import _lib
 
     o = oracle
