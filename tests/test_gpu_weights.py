@@ -56,7 +56,7 @@ class Holder:
         self.transformer = transformer
 
 
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits", [3, 4, 5, 6, 8])
 def test_quantize_on_the_fly_then_save_and_reload(tmp_path, oracle, bits):
     import numpy as np
 
@@ -87,7 +87,7 @@ def test_quantize_on_the_fly_then_save_and_reload(tmp_path, oracle, bits):
     W.save_model(Holder(model), bits, tmp_path, Definition)
 
     # reload without a request, and with a conflicting one
-    for requested in (None, 12 - bits):
+    for requested in (None, 8 if bits == 4 else 4):
         loaded = W.load_saved(Definition, tmp_path)
         fresh = Tower().to(device="cuda", dtype=torch.bfloat16)
         assert W.WeightApplier.apply_and_quantize(loaded, {"transformer": fresh}, requested, Definition) == bits
