@@ -25,7 +25,8 @@
  *     laid end to end.  scales and biases hold one value per `group_size`
  *     consecutive elements of a row.
  *   - bits: 3, 4, 5, 6, 8 for quantize / dequantize / dequantize_rows (3, 5, 6
- *     for 16-bit inputs only); 4 and 8 for qmm_t (MFQ_EUNSUPPORTED otherwise:
+ *     for 16-bit inputs only); 4 and 8 for qmm_t, and 3, 5, 6 for qmm_t with
+ *     one activation row and K <= 8192 (MFQ_EUNSUPPORTED otherwise:
  *     dequantize and use a plain GEMM).
  */
 #ifndef MFQ_H

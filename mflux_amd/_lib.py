@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmfq.so")
 
 F32, F16, BF16 = 0, 1, 2
+MFQ_EUNSUPPORTED = -8  # no kernel for this combination of arguments
 
 # every symbol include/mfq.h declares, with its ctypes signature
 _I64, _INT, _PTR = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p

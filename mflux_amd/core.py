@@ -283,17 +283,28 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
             raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
         bias = bias.to(compute).contiguous()
     w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    lib = _lib.load()
     if bits not in MATMUL_KERNEL_BITS:
-        # 3, 5 and 6 bits: the matmul kernels do not unpack these widths.  The
-        # weight is dequantized by this library's kernel (same single rounding
-        # as inside the fused kernels) and multiplied by the BLAS library's
-        # plain GEMM, float32 accumulation; the bias is added after rounding y.
+        # 3, 5 and 6 bits.  One activation row (the adaLN modulation calls) has a
+        # fused kernel; anything else, or a shape that kernel does not take, is
+        # this library's dequantize kernel (same single rounding as inside the
+        # fused kernels) followed by the BLAS library's plain GEMM, float32
+        # accumulation, the bias added after rounding y.
+        if M == 1:
+            with torch.cuda.device(x.device):
+                rc = lib.mfq_qmm_t(
+                    x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+                    _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
+                    y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device),
+                )
+            if rc != _lib.MFQ_EUNSUPPORTED:
+                _lib.check("mfq_qmm_t", rc)
+                return y.reshape(*lead, N)
         w_full = dequantize(w, scales, biases, group_size, bits)
         y = torch.matmul(x2, w_full.t()) if out_dtype == compute else torch.matmul(x2.float(), w_full.float().t())
         if bias is not None:
             y = y + bias.to(y.dtype)
         return y.reshape(*lead, N)
-    lib = _lib.load()
     with torch.cuda.device(x.device):
         # few output tiles (text-stream shapes): K is split across compute units
         # through a float32 scratch, taken from torch's caching allocator on the

@@ -86,7 +86,9 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
                  int y_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
-  if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;  // 3, 5, 6 bits: dequantize, then a plain GEMM
+  // 3, 5, 6 bits: a fused kernel for one activation row only; otherwise the caller dequantizes and uses a plain GEMM
+  const bool odd_bits = bits != 4 && bits != 8;
+  if (odd_bits && M != 1) return MFQ_EUNSUPPORTED;
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
   if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
@@ -94,6 +96,9 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
   if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
   if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
   if (M > 16 && !mfq::aligned16(y)) return MFQ_EALIGN;  // the GEMM writes y in 16-byte pieces
+  if (odd_bits)
+    return mfq::launch_qmv_odd(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                               (hipStream_t)stream);
   if (M <= 16)
     return mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                            (hipStream_t)stream);

@@ -303,6 +303,84 @@ def test_odd_bit_widths_matmul(oracle, bits, M):
     _assert_close(q(to_dev(x, o.BF16)), ref)
 
 
+@pytest.mark.parametrize("bits", [3, 5, 6])
+@pytest.mark.parametrize("gs,K", [(64, 3072), (64, 4096), (64, 8192), (64, 2048), (32, 96), (32, 1056), (128, 6144),
+                                  (64, 8256)])
+def test_odd_bit_widths_single_row_kernel(oracle, bits, gs, K):
+    """3, 5, 6 bits with one activation row: the fused kernel (one to four units
+    of 32 codes per lane, whole and partial last rounds, all group sizes) and,
+    for K = 8256, the first shape beyond it (dequantize + library GEMM)."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    N = 203
+    args = _case(o, 51, 1, K, N, bits, gs=gs)
+    ref = _ref(o, *args, bits, gs)
+    _assert_close(_run(o, *args, bits, gs), ref)
+    x, wq, s, b, bias = args
+    y32 = mflux_amd.quantized_matmul(to_dev(x, o.BF16).float(), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                     group_size=gs, bits=bits, bias=to_dev(bias, o.BF16))
+    assert y32.dtype == torch.float32
+    _assert_close(y32, ref, tol=5e-3)
+
+
+@pytest.mark.parametrize("bits", [3, 5, 6])
+def test_odd_bit_widths_one_hot(oracle, bits):
+    """One-hot x picks single weights out of the bit stream: every code position
+    of a unit, units of both rounds, against scale * code + bias."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    K, N = 3072, 48
+    w = o.f32_to_bf16_bits(seeded(52, 1, (N, K), 0.02))
+    wq, s, b = o.c_quantize(w, o.BF16, 64, bits)
+    exact = o.dequantize_exact(wq, s, b, o.BF16, 64, bits).astype(np.float64)
+    step = np.abs(o.bf16_bits_to_f32(s).astype(np.float64))
+    for k in list(range(0, 32)) + [32, 63, 64, 1000, 2047, 2048, 2049, 2079, 3040, 3071]:
+        xf = np.zeros((1, K), dtype=np.float32)
+        xf[0, k] = 1.0
+        y = mflux_amd.quantized_matmul(to_dev(o.f32_to_bf16_bits(xf), o.BF16).float(), u32_to_dev(wq),
+                                       to_dev(s, o.BF16), to_dev(b, o.BF16), group_size=64, bits=bits)
+        got = y.cpu().numpy()[0].astype(np.float64)
+        assert np.all(np.abs(got - exact[:, k]) <= 1e-3 * step[:, k // 64]), (bits, k)
+
+
+def test_odd_bit_widths_c_abi_coverage(oracle):
+    """mfq_qmm_t takes 3-, 5- and 6-bit weights for one activation row with rows
+    of at most 8192 codes, and says MFQ_EUNSUPPORTED for anything else."""
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    for bits in (3, 5, 6):
+        for M, K, expect in ((1, 3072, 0), (2, 3072, _lib.MFQ_EUNSUPPORTED), (1, 8256, _lib.MFQ_EUNSUPPORTED)):
+            x, wq, s, b, _ = _case(o, 53, M, K, 16, bits, gs=32, with_bias=False)
+            xd, wd, sd, bd = to_dev(x, o.BF16), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16)
+            y = torch.empty((M, 16), dtype=torch.bfloat16, device="cuda")
+            rc = lib.mfq_qmm_t(xd.data_ptr(), _lib.BF16, M, K, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), _lib.BF16,
+                               None, 16, 32, bits, y.data_ptr(), _lib.BF16, None)
+            torch.cuda.synchronize()
+            assert rc == expect, (bits, M, K, rc)
+
+
+def test_odd_bit_widths_single_row_f16(oracle):
+    import mflux_amd
+    from gpu_util import raw
+
+    o = oracle
+    torch.manual_seed(5)
+    for bits in (3, 5, 6):
+        x = torch.randn(1, 3072, device="cuda").to(torch.float16)
+        w = (torch.randn(130, 3072, device="cuda") * 0.02).to(torch.float16)
+        wq, s, b = mflux_amd.quantize(w, 64, bits)
+        y = mflux_amd.quantized_matmul(x, wq, s, b, bits=bits)
+        ref = o.quantized_matmul_f64(x.double().cpu().numpy(), raw(wq), raw(s), raw(b), o.F16, 64, bits)
+        _assert_close(y, ref)
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 32), (8, 32), (4, 128), (8, 128)])
 def test_qmm_group_sizes(oracle, bits, gs):
     o = oracle
