@@ -114,7 +114,7 @@ def cpu_baseline(torch, x, wq, s, b, sample_rows):
     t0 = time.perf_counter()
     o.c_qmm_t(xs, o.BF16, wq_h, s_h, b_h, o.BF16, None, GS, BITS, threads=threads)
     t_all = time.perf_counter() - t0
-    one_rows = max(1, sample_rows // 8)
+    one_rows = max(1, min(64, sample_rows // 8))
     t0 = time.perf_counter()
     o.c_qmm_t(xs[:one_rows], o.BF16, wq_h, s_h, b_h, o.BF16, None, GS, BITS, threads=1)
     t_one = time.perf_counter() - t0
@@ -137,7 +137,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-rows", type=int, default=512)
+    ap.add_argument("--cpu-sample-rows", type=int, default=2304)
     ap.add_argument("--no-secondary", action="store_true",
                     help="skip the GEMV and quantize measurements (they replay HIP graphs)")
     ap.add_argument("--calibration-copy", action="store_true",
