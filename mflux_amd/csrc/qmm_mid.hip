@@ -141,10 +141,9 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   // loads in flight.  q: k step inside the item (steps past the end repeat the
   // last one and are never consumed).
   // sel: -1, or the Period set to refill with the period that step q starts.
-  auto load = [&](auto sel, Stage& g, int q) __attribute__((always_inline)) {
+  auto load_rest = [&](auto sel, Stage& g, int q) __attribute__((always_inline)) {  // everything but x
     constexpr int kSel = decltype(sel)::value;
     const int k0 = kb + min(q, steps - 1) * TK;
-    // in the order publishing consumes them
     if constexpr (kFast) {
       if constexpr (kSel >= 0) {
         const int g0 = (k0 / GS) & ~3;
@@ -169,8 +168,15 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
         for (int e = 0; e < 4; ++e) g.w[4 * l + e] = v[e];
       }
     }
+  };
+  auto load_x_piece = [&](Stage& g, int q, int i) __attribute__((always_inline)) {
+    const int k0 = kb + min(q, steps - 1) * TK;
+    g.x[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k0 * 2 + xoff[i]);
+  };
+  auto load = [&](auto sel, Stage& g, int q) __attribute__((always_inline)) {
+    load_rest(sel, g, q);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) g.x[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k0 * 2 + xoff[i]);
+    for (int i = 0; i < 4; ++i) load_x_piece(g, q, i);
   };
   // the Period set step e of the unrolled sequence refills, if it starts a period
   auto sel_of = [](auto e) {
@@ -223,8 +229,8 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   // Step e of the unrolled sequence, k step p of the item: the matrix work on
   // buffer e%2, with quarter `sub` of publishing step p+1 to the other buffer
   // in the shadow of the matrix instructions of sub-step `sub` (a scheduling
-  // barrier between sub-steps keeps the interleaving), then the loads of step
-  // p+3 into the registers just published.
+  // barrier between sub-steps keeps the interleaving) and each quarter's
+  // registers refilled for step p+3 as soon as they have been published.
   auto step = [&](auto e, int p) __attribute__((always_inline)) {
     constexpr int kE = decltype(e)::value;
     constexpr int buf = kE & 1;
@@ -251,9 +257,11 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(af[sub & 1][j], bf[sub & 1][i], acc[i][j]);
       publish_part(next, sub, sc, bi, buf ^ 1);
+      // the registers just published are refilled for step p+3 right away
+      load_x_piece(st[buf ^ 1], p + 3, sub);
+      if (sub == 3) load_rest(sel_of(std::integral_constant<int, kE + 3>{}), st[buf ^ 1], p + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
-    load(sel_of(std::integral_constant<int, kE + 3>{}), st[buf ^ 1], p + 3);
     __syncthreads();
   };
 
