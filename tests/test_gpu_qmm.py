@@ -593,3 +593,44 @@ def test_transpose_false_and_input_gradient(oracle, bits):
     assert a.grad is not None and bl.grad is not None and q.weight.grad is None
     # and no autograd graph is built when nothing requires grad
     assert not q(to_dev(x, o.BF16)).requires_grad
+
+
+def test_calls_replay_in_a_hip_graph(oracle):
+    """The kernels take everything from their arguments and the current stream
+    (no memsets, no host synchronisation), so a sequence of calls can be
+    captured once and replayed: one activation row, the medium-M kernel with
+    its K cut (workspace from the capture's allocator) and the large-M kernel,
+    replayed with eager work and synchronisations in between, every replay
+    equal to the eager results bit for bit."""
+    import mflux_amd
+
+    torch.manual_seed(9)
+    shapes = ((1, 3072, 1024, 8), (300, 2048, 520, 4), (2200, 512, 2304, 4))
+    ops = []
+    for M, K, N, bits in shapes:
+        x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+        w = (torch.randn(N, K, device="cuda") * 0.02).to(torch.bfloat16)
+        ops.append((x, *mflux_amd.quantize(w, 64, bits), bits))
+    run = lambda: [mflux_amd.quantized_matmul(x, wq, s, b, bits=bits) for x, wq, s, b, bits in ops]
+    eager = run()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run()
+    for i in range(3):
+        for o in outs:
+            o.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(outs, eager):
+            assert torch.equal(o, e), i
+        # eager work between replays
+        again = run()
+        torch.cuda.synchronize()
+        for a, e in zip(again, eager):
+            assert torch.equal(a, e)
