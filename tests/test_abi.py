@@ -92,7 +92,8 @@ def test_argument_validation_needs_no_device():
     assert call(wq=None) == E["null"]
     assert call(x=base + 4) == E["align"]
     assert call(gs=16) == E["group"]
-    assert call(bits=5) == -8                        # 3, 5, 6 bits: no fused matmul kernel
+    assert call(bits=5) == -8                        # 3, 5, 6 bits: a fused kernel for one activation row only
+    assert call(bits=5, M=1, K=100) == E["shape"]    # ... which validates its arguments like the others
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
