@@ -40,10 +40,12 @@ def _ref(o, x, wq, s, b, bias, bits, gs=64):
     return o.quantized_matmul_f64(xf, wq, s, b, o.BF16, gs, bits, bias_f64=bf)
 
 
-def _assert_close(y: torch.Tensor, ref: np.ndarray, tol=TOL):
+def _assert_close(y: torch.Tensor, ref: np.ndarray, tol=TOL, row_floor=None):
     got = y.detach().to(torch.float64).cpu().numpy()
     assert got.shape == ref.shape
     row_inf = np.abs(ref).max(axis=-1, keepdims=True)
+    if row_floor is not None:
+        row_inf = np.maximum(row_inf, row_floor)
     err = np.abs(got - ref) / np.maximum(row_inf, 1e-30)
     worst = float(err.max())
     assert worst <= tol, f"max |err| / ||row||inf = {worst:.4g} > {tol}"
@@ -634,3 +636,35 @@ def test_calls_replay_in_a_hip_graph(oracle):
         torch.cuda.synchronize()
         for a, e in zip(again, eager):
             assert torch.equal(a, e)
+
+
+def _sweep_cases():
+    """Seeded shapes that sit on and around the borders between the kernels: the
+    row counts where the matvec kernels hand over to each other and to the GEMMs,
+    ragged N (odd, below one tile, just past a tile) and K from one group up."""
+    rng = np.random.default_rng(20240611)
+    m_pool = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 33, 63, 64, 65, 127, 128, 129, 130, 255, 257, 511, 513, 700, 1025]
+    cases = []
+    for i in range(56):
+        gs = int(rng.choice([32, 64, 128]))
+        bits = int(rng.choice([4, 8, 4, 8, 3, 5, 6]))
+        M = int(rng.choice(m_pool))
+        if bits in (3, 5, 6) and M > 64:
+            M = int(rng.choice([1, 1, 2, 40]))
+        K = gs * int(rng.integers(1, 2560 // gs + 1))
+        N = int(rng.choice([1, 3, 8, 17, 64, 100, 127, 128, 129, 255, 256, 264, 391, 520, 641]))
+        cases.append((i, M, K, N, bits, gs))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: "case%d-M%d-K%d-N%d-w%d-g%d" % c)
+def test_shape_sweep_against_oracle(oracle, case):
+    o = oracle
+    i, M, K, N, bits, gs = case
+    args = _case(o, 400 + i, M, K, N, bits, gs=gs, with_bias=bool(i % 2))
+    # The bound is relative to a row's largest output.  With one or three output
+    # features that largest output can itself be next to nothing (a chance
+    # cancellation), so it is held at the size an output of this row has on
+    # average, |x row|_2 times the weights' standard deviation.
+    x_norm = np.linalg.norm(o.bf16_bits_to_f32(args[0]).astype(np.float64), axis=-1, keepdims=True)
+    _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs), row_floor=0.02 * x_norm)
