@@ -155,6 +155,41 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  int group_size, int bits, void* y, int y_dtype, void* workspace,
                  size_t workspace_bytes, void* stream);
 
+/*
+ * A quantized linear layer with LoRA adapters on it in one call:
+ *   y = x @ dequantize(wq, scales, biases)^T + t @ bs^T (+ bias).
+ * Replaces the body of LoRALinear.__call__
+ * (src/mflux/models/common/lora/layer/linear_lora_layer.py:50-53:
+ * base_out + scale * ((x @ lora_A) @ lora_B)) and of FusedLoRALinear.__call__
+ * (src/mflux/models/common/lora/layer/fused_linear_lora_layer.py:13-20, the sum
+ * over several adapters) around a QuantizedLinear base.  The caller passes
+ *   t  [M, rank] = x @ [lora_A_1 | lora_A_2 | ...]      (a plain small GEMM)
+ *   bs [N, rank] = [scale_1 * lora_B_1^T | scale_2 * lora_B_2^T | ...]
+ * both row-major and 16-byte aligned, in x_dtype, with rank (the sum of the
+ * adapters' ranks) zero-padded to a multiple of 16, at most 1024.  The
+ * 256 x 256-tile GEMM treats them as `rank` more k after the layer's own, in
+ * the same float32 accumulators, so the product is rounded once (the
+ * reference rounds the base output, both LoRA products, the scaling and the
+ * sum separately); behind the other kernels a second kernel adds the update
+ * to the rounded product (mfq_low_rank_add).  rank == 0 (t, bs ignored) is
+ * mfq_qmm_t_ws; everything else is as documented there, odd bit widths for
+ * M = 1 included.
+ */
+int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
+                       const void* scales, const void* biases, int sb_dtype, const void* bias,
+                       int64_t N, int group_size, int bits, const void* t, const void* bs,
+                       int64_t rank, void* y, int y_dtype, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
+ * y[M, N] += t[M, rank] @ bs[N, rank]^T in float32, rounded to y_dtype (dtype
+ * or MFQ_F32): the same adapters (see mfq_qmm_t_low_rank for t and bs) behind
+ * a product that did not come from mfq_qmm_t_low_rank, e.g. an odd bit width
+ * with M > 1 that the caller dequantized and multiplied with a library GEMM.
+ */
+int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank,
+                     void* y, int y_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -222,25 +222,53 @@ class _QuantizedMatmulFunction(torch.autograd.Function):
 
 def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
                      transpose: bool = True, group_size: int = 64, bits: int = 4, mode: str = "affine",
-                     *, bias: torch.Tensor | None = None) -> torch.Tensor:
+                     *, bias: torch.Tensor | None = None,
+                     low_rank: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
     """``x @ dequantize(w).T`` (``transpose=True``) or ``x @ dequantize(w)``; see
     ``_quantized_matmul_forward``.  Differentiable with respect to ``x`` and
-    ``bias``."""
+    ``bias``; ``low_rank`` (inference only) is described there."""
     _check_mode("quantized_matmul", mode)
     _check_group_bits("quantized_matmul", group_size, bits)
     if not transpose:
-        if bias is not None:
-            raise ValueError("[quantized_matmul] bias is only fused for transpose=True")
+        if bias is not None or low_rank is not None:
+            raise ValueError("[quantized_matmul] bias and low_rank are only fused for transpose=True")
         return _matmul_untransposed(x, w, scales, biases, group_size, bits)
     needs_grad = torch.is_grad_enabled() and (x.requires_grad or (bias is not None and bias.requires_grad))
     if needs_grad:
+        if low_rank is not None:
+            raise ValueError("[quantized_matmul] low_rank is not differentiable: add the LoRA branch as separate "
+                             "matmuls when gradients are needed")
         return _QuantizedMatmulFunction.apply(x, w, scales, biases, bias, group_size, bits)
-    return _quantized_matmul_forward(x, w, scales, biases, group_size, bits, bias)
+    return _quantized_matmul_forward(x, w, scales, biases, group_size, bits, bias, low_rank)
+
+
+def _low_rank_operands(low_rank, lead: tuple, M: int, N: int, compute: torch.dtype):
+    """Checks ``(t, bs)`` against the product's shape; returns them as contiguous
+    ``[M, R]`` / ``[N, R]`` matrices in the compute dtype."""
+    t, bs = low_rank
+    if t.ndim < 1 or tuple(t.shape[:-1]) != lead or bs.ndim != 2 or bs.shape[0] != N or bs.shape[1] != t.shape[-1]:
+        raise ValueError(f"[quantized_matmul] low_rank must be (t [..., R], bs [{N}, R]) with t's leading "
+                         f"dimensions {lead}; got {tuple(t.shape)} and {tuple(bs.shape)}")
+    R = bs.shape[1]
+    if R == 0 or R % 16 or R > 1024:
+        raise ValueError(f"[quantized_matmul] the low rank must be a multiple of 16 up to 1024 (pad with zeros), got {R}")
+    _require_hip("quantized_matmul", t, "low_rank t")
+    _require_hip("quantized_matmul", bs, "low_rank bs")
+    return t.reshape(M, R).to(compute).contiguous(), bs.to(compute).contiguous(), R
 
 
 def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
-                              group_size: int, bits: int, bias: torch.Tensor | None) -> torch.Tensor:
+                              group_size: int, bits: int, bias: torch.Tensor | None,
+                              low_rank: tuple[torch.Tensor, torch.Tensor] | None = None) -> torch.Tensor:
     """``x @ dequantize(w).T`` with float32 accumulation.
+
+    ``low_rank = (t, bs)`` (not part of ``mx.quantized_matmul``) adds
+    ``t @ bs.T`` to the product: the LoRA branch of
+    src/mflux/models/common/lora/layer/linear_lora_layer.py:50-53 with
+    ``t = x @ lora_A`` (``[..., R]``) and ``bs = scale * lora_B.T`` (``[N, R]``),
+    several adapters concatenated along ``R``, ``R`` zero-padded to a multiple
+    of 16.  The large-M kernel accumulates it with the product before the one
+    rounding; the other kernels are followed by a small second kernel.
 
     ``x``: ``[..., K]``; ``w``: packed ``[N, K*bits/32]``.  The result has dtype
     ``result_type(x, scales)``; when that is float32 (float32 ``x`` against
@@ -284,6 +312,10 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
         bias = bias.to(compute).contiguous()
     w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
     lib = _lib.load()
+    lr_t = lr_bs = None
+    rank = 0
+    if low_rank is not None:
+        lr_t, lr_bs, rank = _low_rank_operands(low_rank, lead, M, N, compute)
     if bits not in MATMUL_KERNEL_BITS:
         # 3, 5 and 6 bits.  One activation row (the adaLN modulation calls) has a
         # fused kernel; anything else, or a shape that kernel does not take, is
@@ -292,18 +324,25 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
         # accumulation, the bias added after rounding y.
         if M == 1:
             with torch.cuda.device(x.device):
-                rc = lib.mfq_qmm_t(
+                rc = lib.mfq_qmm_t_low_rank(
                     x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
                     _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
-                    y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device),
+                    lr_t.data_ptr() if rank else None, lr_bs.data_ptr() if rank else None, rank,
+                    y.data_ptr(), _DTYPE_CODE[out_dtype], None, 0, _stream_ptr(x.device),
                 )
             if rc != _lib.MFQ_EUNSUPPORTED:
-                _lib.check("mfq_qmm_t", rc)
+                _lib.check("mfq_qmm_t_low_rank", rc)
                 return y.reshape(*lead, N)
         w_full = dequantize(w, scales, biases, group_size, bits)
         y = torch.matmul(x2, w_full.t()) if out_dtype == compute else torch.matmul(x2.float(), w_full.float().t())
         if bias is not None:
             y = y + bias.to(y.dtype)
+        if rank:
+            y = y.contiguous()
+            with torch.cuda.device(x.device):
+                rc = lib.mfq_low_rank_add(lr_t.data_ptr(), lr_bs.data_ptr(), _DTYPE_CODE[compute], M, N, rank,
+                                          y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device))
+            _lib.check("mfq_low_rank_add", rc)
         return y.reshape(*lead, N)
     with torch.cuda.device(x.device):
         # few output tiles (text-stream shapes): K is split across compute units
@@ -311,11 +350,12 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
         # current stream (so its reuse is ordered after this call)
         ws_bytes = lib.mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
-        rc = lib.mfq_qmm_t_ws(
+        rc = lib.mfq_qmm_t_low_rank(
             x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
             _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
+            lr_t.data_ptr() if rank else None, lr_bs.data_ptr() if rank else None, rank,
             y.data_ptr(), _DTYPE_CODE[out_dtype], ws.data_ptr() if ws is not None else None, ws_bytes,
             _stream_ptr(x.device),
         )
-    _lib.check("mfq_qmm_t_ws", rc)
+    _lib.check("mfq_qmm_t_low_rank", rc)
     return y.reshape(*lead, N)

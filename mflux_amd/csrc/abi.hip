@@ -85,7 +85,24 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* 
 int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                  const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
                  int y_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  return mfq_qmm_t_low_rank(x, x_dtype, M, K, wq, scales, biases, sb_dtype, bias, N, group_size, bits, nullptr, nullptr,
+                            0, y, y_dtype, workspace, workspace_bytes, stream);
+}
+
+int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                       const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits,
+                       const void* t, const void* bs, int64_t rank, void* y, int y_dtype, void* workspace,
+                       size_t workspace_bytes, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
+  if (rank < 0 || rank > 1024 || rank % 16) return MFQ_ESHAPE;
+  if (rank && (!t || !bs)) return MFQ_ENULL;
+  if (rank && (!mfq::aligned16(t) || !mfq::aligned16(bs))) return MFQ_EALIGN;
+  mfq::LowRank low_rank;
+  if (rank) {
+    low_rank.t = t;
+    low_rank.bs = bs;
+    low_rank.R = (int)rank;
+  }
   // 3, 5, 6 bits: a fused kernel for one activation row only; otherwise the caller dequantizes and uses a plain GEMM
   const bool odd_bits = bits != 4 && bits != 8;
   if (odd_bits && M != 1) return MFQ_EUNSUPPORTED;
@@ -96,12 +113,16 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
   if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
   if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
   if (M > 16 && !mfq::aligned16(y)) return MFQ_EALIGN;  // the GEMM writes y in 16-byte pieces
-  if (odd_bits)
-    return mfq::launch_qmv_odd(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
-                               (hipStream_t)stream);
-  if (M <= 16)
-    return mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
-                           (hipStream_t)stream);
+  if (odd_bits) {
+    const int rc = mfq::launch_qmv_odd(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                       (hipStream_t)stream);
+    return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
+  }
+  if (M <= 16) {
+    const int rc = mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                   (hipStream_t)stream);
+    return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
+  }
   if (K % 64) {
     // group size 32 with K an odd multiple of it: the matrix-core GEMM steps k
     // by 64, so these rare shapes go through the small-M kernel 16 rows at a time
@@ -113,10 +134,25 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                                      (hipStream_t)stream);
       if (rc) return rc;
     }
-    return MFQ_OK;
+    return mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
   }
   return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, workspace,
-                         workspace_bytes, (hipStream_t)stream);
+                         workspace_bytes, (hipStream_t)stream, low_rank);
+}
+
+int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank, void* y, int y_dtype,
+                     void* stream) {
+  if (!is16(dtype)) return MFQ_EDTYPE;
+  if (y_dtype != dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
+  if (M <= 0 || N <= 0 || M > INT32_MAX || N > INT32_MAX) return MFQ_ESHAPE;
+  if (rank <= 0 || rank > 1024 || rank % 16) return MFQ_ESHAPE;
+  if (!t || !bs || !y) return MFQ_ENULL;
+  if (!mfq::aligned16(t) || !mfq::aligned16(bs)) return MFQ_EALIGN;
+  mfq::LowRank low_rank;
+  low_rank.t = t;
+  low_rank.bs = bs;
+  low_rank.R = (int)rank;
+  return mfq::launch_low_rank_add(dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

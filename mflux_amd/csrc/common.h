@@ -152,6 +152,16 @@ inline int compute_units() {
   return n;
 }
 
+// A low-rank update added to a product, y += t @ bs^T: t [M, R] holds the
+// activations already multiplied by the LoRA down-projections, bs [N, R] the
+// scaled up-projections, both row-major in the activation's 16-bit type, R a
+// multiple of 16 (zero-padded).  R == 0: no update.
+struct LowRank {
+  const void* t = nullptr;
+  const void* bs = nullptr;
+  int R = 0;
+};
+
 // Entry points of the individual translation units (host side).
 int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, int bits, uint32_t* wq,
                     void* scales, void* biases, hipStream_t stream);
@@ -175,9 +185,13 @@ int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32
                     hipStream_t stream);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
+// low_rank: added inside the 256 x 256-tile kernel's epilogue, by a second
+// kernel after the other ones
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               void* workspace, size_t workspace_bytes, hipStream_t stream);
+               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
+// y[M, N] += t @ bs^T, rounded to y's type (dtype: the type of t, bs and a 16-bit y)
+int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream);
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // the 128 x 128-tile kernel for a few hundred activation rows (K % 64 == 0)
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,

@@ -148,11 +148,12 @@ __host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, 
   n0 = (in_band / band_rows) * BN;
 }
 
-template <typename T, int GS, int BITS, bool kFast>
+template <typename T, int GS, int BITS, bool kFast, bool kLowRank>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
-    int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits, float* __restrict__ planes) {
+    int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits, float* __restrict__ planes,
+    const uint16_t* __restrict__ lr_t, const uint16_t* __restrict__ lr_bs, int lr_rank) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   using WR = WeightRegs<T, GS, BITS>;
@@ -418,6 +419,44 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       for (int c = 0; c < 7; ++c) dq_chunk(wa, j, 0, c, d, bf[j]);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // The low-rank update (kLowRank): lr_rank more k after the item's own, whose
+  // x side is lr_t [M, lr_rank] and whose weight side is lr_bs [N, lr_rank],
+  // both 16-bit and unquantised.  They are few, so they bypass the pipeline: a
+  // lane's 8 consecutive k of a row are one 16-byte load straight into a matrix
+  // fragment (k 16 c + 8 h + 0..7 for chunk c of 16, the same for both sides).
+  auto low_rank_steps = [&](int m0, int n0) {
+    int lane_e = lane;  // opaque copy, see store_tile_staged
+    asm volatile("" : "+v"(lane_e));
+    const int r = lane_e & 31;
+    const int h = lane_e >> 5;
+    const char* tb = reinterpret_cast<const char*>(lr_t) + 16 * h;
+    const char* bb = reinterpret_cast<const char*>(lr_bs) + 16 * h;
+    const uint32_t pitch = (uint32_t)lr_rank * 2u;  // bytes per row of either matrix
+    uint32_t boff[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) boff[j] = (uint32_t)min(n0 + wn + 32 * j + r, N - 1) * pitch;
+    const uint32_t toff = (uint32_t)min(m0 + r, M - 1) * pitch;
+    // rows 32 ai + r of the tile: 32 * pitch apart until the clamp at M - 1
+    const uint32_t t_last = (uint32_t)(M - 1) * pitch;
+#pragma unroll 1
+    for (uint32_t kb = 0; kb < pitch; kb += 32) {
+      vec8 wf[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) wf[j] = *reinterpret_cast<const vec8*>(bb + boff[j] + kb);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        vec8 xf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          xf[i] = *reinterpret_cast<const vec8*>(tb + min(toff + (uint32_t)(4 * half + i) * 32u * pitch, t_last) + kb);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[4 * half + i][j] = mfma32(wf[j], xf[i], acc[4 * half + i][j]);
+      }
+    }
   };
 
   // Writes the finished tile.  The weights were the matrix instruction's A
@@ -702,6 +741,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
       if (step < steps) do_step(even_step, keep, wa, wb, (steps - 1) * BK, 0, 0);
     }
+    if constexpr (kLowRank) {
+      if (item.first_step == 0) low_rank_steps(m0, n0);  // once per tile: by the item that has its first k range
+    }
     store_tile(m0, n0);
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -830,10 +872,11 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
   }
 }
 
-template <typename T, int GS, int BITS, bool kFast>
+template <typename T, int GS, int BITS, bool kFast, bool kLowRank = false>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                  const void* bias, int64_t N, void* y, int y_dtype, TailPlan plan, void* planes, hipStream_t stream) {
-  auto kernel = qmm_kernel<T, GS, BITS, kFast>;
+                  const void* bias, int64_t N, void* y, int y_dtype, TailPlan plan, void* planes, hipStream_t stream,
+                  LowRank lr = LowRank()) {
+  auto kernel = qmm_kernel<T, GS, BITS, kFast, kLowRank>;
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -849,7 +892,7 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
                      (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.n_whole, plan.splits,
-                     (float*)planes);
+                     (float*)planes, (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R);
   if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
   if (plan.splits > 1) {
     const unsigned blocks = (unsigned)n_tail * (BM * BN / 4 / 256);
@@ -869,9 +912,10 @@ inline size_t tail_plane_bytes(int64_t M, int64_t N, TailPlan plan) {
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
-               hipStream_t stream) {
+               hipStream_t stream, LowRank lr) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
+  if ((M + BM) * lr.R >= (int64_t)1 << 31 || (N + BN) * lr.R >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
   const TailPlan whole{(int)tiles, 1};
   // period-wise scale loads: whole periods, at least two pairs of steps, and
@@ -879,30 +923,41 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   const int64_t steps = K / BK;
   constexpr int kPer = ScaleRegs<T, GS>::kPeriod;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
-  if (!(steps % kPer == 0 && steps >= 4 && aligned8))
-    return launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, whole, nullptr, stream);
+  if (!(steps % kPer == 0 && steps >= 4 && aligned8)) {
+    // the rare shapes without period-wise scale loads: the update comes from its own kernel
+    const int rc =
+        launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, whole, nullptr, stream);
+    return rc ? rc : launch_low_rank_add(T::code, lr, M, N, y, y_dtype, stream);
+  }
   TailPlan plan = plan_tail(M, N, K, kPer, compute_units());
   if (plan.splits > 1 && (!workspace || workspace_bytes < tail_plane_bytes(M, N, plan) || !aligned16(workspace)))
     plan = whole;
+  if (lr.R)
+    return launch_kernel<T, GS, BITS, true, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, workspace,
+                                                  stream, lr);
   return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, workspace, stream);
 }
 
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                 const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-                hipStream_t stream) {
-  if (bits == 4) return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
-  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
+                hipStream_t stream, LowRank lr) {
+  if (bits == 4)
+    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
 }
 
 template <typename T>
 int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
               const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-              hipStream_t stream) {
+              hipStream_t stream, LowRank lr) {
   switch (gs) {
-    case 32: return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
-    case 64: return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
-    default: return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    case 32:
+      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+    case 64:
+      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+    default:
+      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
   }
 }
 
@@ -943,16 +998,18 @@ int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, i
 
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               void* workspace, size_t workspace_bytes, hipStream_t stream) {
-  if (use_mid_kernel(M, N, K))
-    return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
-                          workspace_bytes, stream);
+               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+  if (use_mid_kernel(M, N, K)) {
+    const int rc = launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
+                                  workspace_bytes, stream);
+    return rc ? rc : launch_low_rank_add(dtype, low_rank, M, N, y, y_dtype, stream);
+  }
   if (dtype == MFQ_BF16)
     return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                           stream);
+                           stream, low_rank);
   if (dtype == MFQ_F16)
     return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                          stream);
+                          stream, low_rank);
   return MFQ_EDTYPE;
 }
 

@@ -1,0 +1,121 @@
+"""LoRA adapters on (quantized) linear layers.
+
+Mirrors mflux's wrappers, same names and attributes:
+``LoRALinear`` (src/mflux/models/common/lora/layer/linear_lora_layer.py:8-53:
+``from_linear(linear, r, scale)``, ``linear``, ``scale``, ``lora_A [K, r]``,
+``lora_B [r, N]``, ``base + scale * (x @ A) @ B``) and ``FusedLoRALinear``
+(src/mflux/models/common/lora/layer/fused_linear_lora_layer.py:7-20:
+``base_linear``, ``loras``, the sum over the adapters).
+
+Around a ``QuantizedLinear`` base on the GPU, at inference, the whole layer is
+one call of the quantized matmul: the adapters' down-projections are
+concatenated into one ``[K, R]`` matrix (one small GEMM gives ``t = x @ A``),
+the scaled up-projections into one ``[N, R]`` matrix, and the kernel treats
+them as ``R`` more ``k`` of the same product.  When gradients are needed, or
+the base is not quantized, the layer is the reference's composition of
+separate matmuls.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import core
+from .nn import Linear, QuantizedLinear
+
+_RANK_STEP = 16  # the kernels take the low rank in steps of 16
+
+
+class LoRALinear(torch.nn.Module):
+    @staticmethod
+    def from_linear(linear: torch.nn.Module, r: int = 16, scale: float = 1.0) -> "LoRALinear":
+        output_dims, input_dims = linear.weight.shape
+        if isinstance(linear, QuantizedLinear):
+            # packed words -> elements (the reference multiplies by 32 // bits, which is only right for 4 and 8 bits)
+            input_dims = input_dims * 32 // linear.bits
+        ref = linear.scales if isinstance(linear, QuantizedLinear) else linear.weight
+        lora_lin = LoRALinear(input_dims=input_dims, output_dims=output_dims, r=r, scale=scale, device=ref.device,
+                              dtype=ref.dtype, _make_linear=False)
+        lora_lin.linear = linear
+        return lora_lin
+
+    def __init__(self, input_dims: int, output_dims: int, r: int = 8, scale: float = 1.0, bias: bool = False, *,
+                 device=None, dtype: torch.dtype = torch.bfloat16, _make_linear: bool = True):
+        super().__init__()
+        if _make_linear:
+            self.linear = Linear(input_dims, output_dims, bias=bias, device=device, dtype=dtype)
+        self.scale = scale
+        bound = 1 / math.sqrt(input_dims)
+        make = lambda *shape: torch.nn.Parameter(
+            torch.empty(shape, device=device, dtype=torch.float32).uniform_(-bound, bound).to(dtype))
+        self.lora_A = make(input_dims, r)
+        self.lora_B = make(r, output_dims)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _forward(self, self.linear, [self], x)
+
+
+class FusedLoRALinear(torch.nn.Module):
+    def __init__(self, base_linear: torch.nn.Module, loras: list[LoRALinear]):
+        super().__init__()
+        self.base_linear = base_linear
+        self.loras = torch.nn.ModuleList(loras)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _forward(self, self.base_linear, list(self.loras), x)
+
+
+def _composed(base: torch.nn.Module, loras: list[LoRALinear], x: torch.Tensor) -> torch.Tensor:
+    """The reference's arithmetic: separate matmuls, every intermediate rounded."""
+    out = base(x)
+    if len(loras) == 1:
+        lora = loras[0]
+        return out + lora.scale * torch.matmul(torch.matmul(x.to(lora.lora_A.dtype), lora.lora_A), lora.lora_B)
+    lora_out = torch.zeros_like(out)
+    for lora in loras:
+        lora_out = lora_out + lora.scale * torch.matmul(torch.matmul(x.to(lora.lora_A.dtype), lora.lora_A),
+                                                        lora.lora_B)
+    return out + lora_out
+
+
+def pack_adapters(loras: list[LoRALinear], dtype: torch.dtype) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(a_cat [K, R], bs [N, R])`` for ``quantized_matmul(..., low_rank=(x @ a_cat, bs))``:
+    the down-projections side by side and the up-projections, scaled in float32
+    and transposed, side by side, ``R`` = the sum of the ranks rounded up to a
+    multiple of 16 with zero columns."""
+    a_cat = torch.cat([lora.lora_A.detach().to(dtype) for lora in loras], dim=1)
+    bs = torch.cat([(float(lora.scale) * lora.lora_B.detach().float()).t() for lora in loras], dim=1).to(dtype)
+    pad = -a_cat.shape[1] % _RANK_STEP
+    if pad:
+        a_cat = torch.nn.functional.pad(a_cat, (0, pad))
+        bs = torch.nn.functional.pad(bs, (0, pad))
+    return a_cat.contiguous(), bs.contiguous()
+
+
+def _packed_for(owner: torch.nn.Module, loras: list[LoRALinear], dtype: torch.dtype):
+    # rebuilt when an adapter's tensors are replaced or written in place, or a scale changes
+    key = (dtype,) + tuple((id(lora), lora.lora_A.data_ptr(), lora.lora_A._version, lora.lora_B.data_ptr(),
+                            lora.lora_B._version, float(lora.scale)) for lora in loras)
+    cache = owner.__dict__.get("_packed_adapters")
+    if cache is None or cache[0] != key:
+        cache = (key, pack_adapters(loras, dtype))
+        owner.__dict__["_packed_adapters"] = cache
+    return cache[1]
+
+
+def _forward(owner: torch.nn.Module, base: torch.nn.Module, loras: list[LoRALinear], x: torch.Tensor) -> torch.Tensor:
+    if not loras:
+        return base(x)
+    needs_grad = torch.is_grad_enabled() and (
+        x.requires_grad or any(lora.lora_A.requires_grad or lora.lora_B.requires_grad for lora in loras))
+    rank = sum(lora.lora_A.shape[1] for lora in loras)
+    fused = (isinstance(base, QuantizedLinear) and x.is_cuda and not needs_grad and rank <= 1024
+             and base.scales.dtype in (torch.bfloat16, torch.float16) and x.numel() > 0)
+    if not fused:
+        return _composed(base, loras, x)
+    compute = base.scales.dtype
+    a_cat, bs = _packed_for(owner, loras, compute)
+    t = torch.matmul(x.to(compute), a_cat)
+    return core.quantized_matmul(x, base.weight, base.scales, base.biases, transpose=True, group_size=base.group_size,
+                                 bits=base.bits, mode=base.mode, bias=base.bias, low_rank=(t, bs))

@@ -20,7 +20,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
-                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes"):
+                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add"):
         assert must in names
 
 
@@ -94,6 +94,29 @@ def test_argument_validation_needs_no_device():
     assert call(gs=16) == E["group"]
     assert call(bits=5) == -8                        # 3, 5, 6 bits: a fused kernel for one activation row only
     assert call(bits=5, M=1, K=100) == E["shape"]    # ... which validates its arguments like the others
+
+    # the LoRA entry points: the rank comes in steps of 16 with both matrices present and aligned
+    lr = lib.mfq_qmm_t_low_rank
+
+    def call_lr(t=base, bs=base, rank=16, **kw):
+        a = {**args, **kw}
+        return lr(a["x"], a["xd"], a["M"], a["K"], a["wq"], a["s"], a["b"], a["sd"], a["bias"], a["N"], a["gs"],
+                  a["bits"], t, bs, rank, a["y"], a["yd"], None, 0, a["stream"])
+
+    assert call_lr(rank=8) == E["shape"]
+    assert call_lr(rank=-16) == E["shape"]
+    assert call_lr(rank=2048) == E["shape"]
+    assert call_lr(t=None) == E["null"]
+    assert call_lr(bs=base + 2) == E["align"]
+    assert call_lr(K=100) == E["shape"]
+    assert call_lr(rank=0, t=None, bs=None, wq=None) == E["null"]   # rank 0: the plain call's checks
+    add = lib.mfq_low_rank_add
+    assert add(base, base, _lib.F32, 4, 8, 16, base, _lib.F32, None) == E["dtype"]
+    assert add(base, base, _lib.BF16, 4, 8, 16, base, _lib.F16, None) == E["dtype"]
+    assert add(base, base, _lib.BF16, 0, 8, 16, base, _lib.BF16, None) == E["shape"]
+    assert add(base, base, _lib.BF16, 4, 8, 24, base, _lib.BF16, None) == E["shape"]
+    assert add(base, None, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["null"]
+    assert add(base + 8, base, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["align"]
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
