@@ -237,6 +237,35 @@ def main():
         library[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
         del w16
 
+    # ---- secondary: a rank-16 LoRA on the two linears --------------------------
+    # the whole layer (x @ A included) as one fused call against the reference's
+    # composition of separate matmuls, and the kernel alone with the update
+    lora = {}
+    for name, x, wq, s, b in (() if args.no_secondary else ops):
+        from mflux_amd.lora import LoRALinear, _composed, pack_adapters
+
+        K, N = x.shape[1], wq.shape[0]
+        base = mflux_amd.nn.QuantizedLinear(K, N, bias=False, group_size=GS, bits=BITS)
+        base.weight, base.scales, base.biases = wq, s, b
+        layer = LoRALinear.from_linear(base, r=16, scale=1.0)
+        with torch.no_grad():
+            a_cat, bs = pack_adapters([layer], torch.bfloat16)
+            t = torch.matmul(x, a_cat)
+            calls = {
+                "kernel_with_update_us": lambda: mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=BITS,
+                                                                            low_rank=(t, bs)),
+                "fused_layer_us": lambda: layer(x),
+                "separate_matmuls_us": lambda: _composed(base, [layer], x),
+            }
+            res = {}
+            for key, fn in calls.items():
+                for _ in range(5):
+                    fn()
+                res[key] = round(min(event_ms(fn, 10, torch) for _ in range(3)) * 1e3, 1)
+        res["base_us"] = per_shape[name]["us"]
+        lora[name] = res
+        del base, layer, a_cat, bs, t
+
     # ---- secondary: GEMV of the adaLN modulation shape, cold weights -----------
     gemv = {}
     Kg, Ng = 3072, 18432
@@ -304,7 +333,7 @@ def main():
         "per_shape": per_shape,
         "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "gemv_w8": gemv.get("w8", {}),
                       "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
-                      "library_bf16_gemm_same_operands": library},
+                      "qmm_w4_lora_r16": lora, "library_bf16_gemm_same_operands": library},
     }
     if not args.no_cpu_baseline:
         name, x, wq, s, b = ops[0]

@@ -166,14 +166,14 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
  *   t  [M, rank] = x @ [lora_A_1 | lora_A_2 | ...]      (a plain small GEMM)
  *   bs [N, rank] = [scale_1 * lora_B_1^T | scale_2 * lora_B_2^T | ...]
  * both row-major and 16-byte aligned, in x_dtype, with rank (the sum of the
- * adapters' ranks) zero-padded to a multiple of 16, at most 1024.  The
- * 256 x 256-tile GEMM treats them as `rank` more k after the layer's own, in
- * the same float32 accumulators, so the product is rounded once (the
- * reference rounds the base output, both LoRA products, the scaling and the
- * sum separately); behind the other kernels a second kernel adds the update
- * to the rounded product (mfq_low_rank_add).  rank == 0 (t, bs ignored) is
- * mfq_qmm_t_ws; everything else is as documented there, odd bit widths for
- * M = 1 included.
+ * adapters' ranks) zero-padded to a multiple of 16, at most 1024.  The GEMM
+ * kernels (M > 16) treat them as `rank` more k after the layer's own, in the
+ * same float32 accumulators, so the product is rounded once (the reference
+ * rounds the base output, both LoRA products, the scaling and the sum
+ * separately); behind the matvec kernels (M <= 16) a second kernel adds the
+ * update to the rounded product (mfq_low_rank_add).  rank == 0 (t, bs
+ * ignored) is mfq_qmm_t_ws; everything else is as documented there, odd bit
+ * widths for M = 1 included.
  */
 int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
                        const void* scales, const void* biases, int sb_dtype, const void* bias,

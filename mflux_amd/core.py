@@ -267,8 +267,9 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
     src/mflux/models/common/lora/layer/linear_lora_layer.py:50-53 with
     ``t = x @ lora_A`` (``[..., R]``) and ``bs = scale * lora_B.T`` (``[N, R]``),
     several adapters concatenated along ``R``, ``R`` zero-padded to a multiple
-    of 16.  The large-M kernel accumulates it with the product before the one
-    rounding; the other kernels are followed by a small second kernel.
+    of 16.  The GEMM kernels (more than 16 rows) accumulate it with the product
+    before the one rounding; the matvec kernels are followed by a small second
+    kernel.
 
     ``x``: ``[..., K]``; ``w``: packed ``[N, K*bits/32]``.  The result has dtype
     ``result_type(x, scales)``; when that is float32 (float32 ``x`` against

@@ -185,8 +185,8 @@ int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32
                     hipStream_t stream);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
-// low_rank: added inside the 256 x 256-tile kernel's epilogue, by a second
-// kernel after the other ones
+// low_rank: accumulated with the product by both GEMM kernels (a second kernel
+// adds it after the matvec kernels)
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
@@ -196,7 +196,7 @@ size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // the 128 x 128-tile kernel for a few hundred activation rows (K % 64 == 0)
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                   void* workspace, size_t workspace_bytes, hipStream_t stream);
+                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
 size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // y = sum of `splits` float32 planes of M x N (+ bias), rounded to y's type; dtype is the type of bias and 16-bit y
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,

@@ -5,9 +5,9 @@
 // (src/mflux/models/common/lora/layer/linear_lora_layer.py:50-53, and the sum
 // over several adapters in fused_linear_lora_layer.py:13-20), with
 // t = x @ [A_1 | A_2 | ...] and bs = [scale_1 * B_1^T | scale_2 * B_2^T | ...].
-// The 256 x 256-tile GEMM adds the update inside its own epilogue; this kernel
-// serves the products that come from the other kernels (one to sixteen
-// activation rows, the 128-column-tile GEMM, dequantised odd bit widths).
+// The GEMM kernels accumulate the update with the product themselves; this
+// kernel serves the products that come from elsewhere (one to sixteen
+// activation rows, odd bit widths dequantised for a library GEMM).
 //
 // A workgroup of four wavefronts owns 64 rows x 128 columns of y; wavefront w
 // takes columns [32w, 32w+32) as two 32x32x16 matrix-core accumulators.  R is

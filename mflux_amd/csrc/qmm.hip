@@ -999,11 +999,9 @@ int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, i
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
-  if (use_mid_kernel(M, N, K)) {
-    const int rc = launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
-                                  workspace_bytes, stream);
-    return rc ? rc : launch_low_rank_add(dtype, low_rank, M, N, y, y_dtype, stream);
-  }
+  if (use_mid_kernel(M, N, K))
+    return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
+                          workspace_bytes, stream, low_rank);
   if (dtype == MFQ_BF16)
     return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
                            stream, low_rank);

@@ -65,7 +65,8 @@ template <typename T, int GS, int BITS, bool kFast, int kWavesM>
 __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
-    int N, int K, int tiles_m, int tiles_n, int steps) {
+    int N, int K, int tiles_m, int tiles_n, int steps, const uint16_t* __restrict__ lr_t,
+    const uint16_t* __restrict__ lr_bs, int lr_rank) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   constexpr int TM = tile_m(kWavesM);
@@ -288,6 +289,34 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     if (p < steps) step(std::integral_constant<int, 0>{}, p);
   }
 
+  // ---- low-rank update (lr_rank > 0): lr_rank more k after the item's own,
+  // x side lr_t [M, lr_rank], weight side lr_bs [N, lr_rank], 16-bit and
+  // unquantised.  They are few, so they come straight from memory as matrix
+  // fragments (a lane's 8 consecutive k of a row are one 16-byte load); of the
+  // k ranges of a tile the first one adds them.
+  if (lr_rank > 0 && split == 0) {
+    const uint16_t* trow[2];
+    const uint16_t* brow[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      trow[i] = lr_t + (int64_t)min(m0 + 64 * wm + 32 * i + r, M - 1) * lr_rank + 8 * h;
+      brow[i] = lr_bs + (int64_t)min(n0 + 64 * wn + 32 * i + r, N - 1) * lr_rank + 8 * h;
+    }
+#pragma unroll 1
+    for (int k = 0; k < lr_rank; k += 16) {
+      vec8 wf[2], xf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        wf[i] = *reinterpret_cast<const vec8*>(brow[i] + k);
+        xf[i] = *reinterpret_cast<const vec8*>(trow[i] + k);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(wf[j], xf[i], acc[i][j]);
+    }
+  }
+
   // ---- epilogue: accumulator [i][j], register e holds output row
   // m0 + 64wm + 32i + r and column n0 + 64wn + 32j + 8(e/4) + 4h + e%4.
   // Every LDS tile is free now (the loop ended with a barrier); each wavefront
@@ -419,7 +448,7 @@ inline MidPlan plan_mid(int64_t M, int64_t N, int64_t K, int period, int cus) {
 
 template <typename T, int GS, int BITS, bool kFast, int kWavesM>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                  const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream) {
+                  const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr) {
   auto kernel = qmm_mid_kernel<T, GS, BITS, kFast, kWavesM>;
   constexpr int kLds = lds_bytes(kWavesM);
   static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
@@ -434,35 +463,36 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   const int64_t n_items = (int64_t)tiles_m * tiles_n * plan.splits;
   hipLaunchKernelGGL(kernel, dim3((unsigned)n_items), dim3(threads_of(kWavesM)), kLds, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
-                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.steps);
+                     (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.steps,
+                     (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R);
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 template <typename T, int GS, int BITS, bool kFast>
 int launch_tile(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream) {
+                const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr) {
   if (waves_m_of(M) == 2)
-    return launch_kernel<T, GS, BITS, kFast, 2>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream);
-  return launch_kernel<T, GS, BITS, kFast, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream);
+    return launch_kernel<T, GS, BITS, kFast, 2>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr);
+  return launch_kernel<T, GS, BITS, kFast, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr);
 }
 
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
-               hipStream_t stream) {
+               hipStream_t stream, LowRank lr) {
   const int64_t steps = K / TK;
   constexpr int kPer = 4 * GS / TK;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
   if (!(steps % kPer == 0 && aligned8))
     return launch_tile<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
-                                           stream);
+                                           stream, lr);
   const MidPlan plan = plan_mid(M, N, K, kPer, compute_units());
   const size_t need = (size_t)plan.splits * M * N * sizeof(float);
   if (plan.splits == 1 || !workspace || workspace_bytes < need || !aligned16(workspace))
     return launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
-                                          stream);
+                                          stream, lr);
   if (int rc = launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
-                                              stream))
+                                              stream, lr))
     return rc;
   return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
 }
@@ -470,19 +500,23 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                 const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-                hipStream_t stream) {
-  if (bits == 4) return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
-  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream);
+                hipStream_t stream, LowRank lr) {
+  if (bits == 4)
+    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
 }
 
 template <typename T>
 int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
               const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-              hipStream_t stream) {
+              hipStream_t stream, LowRank lr) {
   switch (gs) {
-    case 32: return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
-    case 64: return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
-    default: return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream);
+    case 32:
+      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+    case 64:
+      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+    default:
+      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
   }
 }
 
@@ -496,15 +530,15 @@ size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
 
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                   void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if (dtype == MFQ_BF16)
     return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                           stream);
+                           stream, low_rank);
   if (dtype == MFQ_F16)
     return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                          stream);
+                          stream, low_rank);
   return MFQ_EDTYPE;
 }
 

@@ -9,7 +9,7 @@ Mirrors mflux's wrappers, same names and attributes:
 
 Around a ``QuantizedLinear`` base on the GPU, at inference, the whole layer is
 one call of the quantized matmul: the adapters' down-projections are
-concatenated into one ``[K, R]`` matrix (one small GEMM gives ``t = x @ A``),
+concatenated into one ``[K, R]`` matrix (one small library GEMM gives ``t = x @ A``),
 the scaled up-projections into one ``[N, R]`` matrix, and the kernel treats
 them as ``R`` more ``k`` of the same product.  When gradients are needed, or
 the base is not quantized, the layer is the reference's composition of
@@ -116,6 +116,7 @@ def _forward(owner: torch.nn.Module, base: torch.nn.Module, loras: list[LoRALine
         return _composed(base, loras, x)
     compute = base.scales.dtype
     a_cat, bs = _packed_for(owner, loras, compute)
+    # the down-projection is a plain skinny GEMM: the BLAS library's split-K kernels run it at memory speed
     t = torch.matmul(x.to(compute), a_cat)
     return core.quantized_matmul(x, base.weight, base.scales, base.biases, transpose=True, group_size=base.group_size,
                                  bits=base.bits, mode=base.mode, bias=base.bias, low_rank=(t, bs))
