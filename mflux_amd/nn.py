@@ -131,6 +131,41 @@ class QuantizedLinear(torch.nn.Module):
         return ql
 
 
+def concat_quantized(layers: list[QuantizedLinear]) -> QuantizedLinear:
+    """One ``QuantizedLinear`` whose output is the outputs of ``layers`` side by
+    side: the packed rows, scales and biases of a weight belong to its output
+    feature alone, so stacking them along N needs no requantization.  The q, k
+    and v projections of an attention block (e.g.
+    src/mflux/models/flux/model/flux_transformer/common/attention_utils.py:21-23,
+    three calls on the same input) become one launch over three times the
+    tiles, which fills the GPU better than three small ones; the caller splits
+    the result with ``split`` / slicing (views, no copy).  The inputs are left
+    untouched (their tensors are copied)."""
+    if not layers:
+        raise ValueError("[concat_quantized] needs at least one layer")
+    first = layers[0]
+    for layer in layers:
+        if not isinstance(layer, QuantizedLinear):
+            raise ValueError(f"[concat_quantized] expected QuantizedLinear layers, got {type(layer).__name__}")
+        if (layer.input_dims, layer.group_size, layer.bits, layer.mode, layer.scales.dtype) != (
+                first.input_dims, first.group_size, first.bits, first.mode, first.scales.dtype):
+            raise ValueError("[concat_quantized] the layers must share input_dims, group_size, bits, mode and dtype")
+    out = QuantizedLinear.__new__(QuantizedLinear)
+    torch.nn.Module.__init__(out)
+    out.group_size, out.bits, out.mode = first.group_size, first.bits, first.mode
+    out.register_buffer("weight", torch.cat([layer.weight for layer in layers], dim=0))
+    out.register_buffer("scales", torch.cat([layer.scales for layer in layers], dim=0))
+    out.register_buffer("biases", torch.cat([layer.biases for layer in layers], dim=0))
+    if any(layer.bias is not None for layer in layers):
+        parts = [layer.bias if layer.bias is not None else
+                 torch.zeros(layer.output_dims, dtype=first.scales.dtype, device=first.scales.device)
+                 for layer in layers]
+        out.register_buffer("bias", torch.cat(parts, dim=0))
+    else:
+        out.bias = None
+    return out
+
+
 class Linear(torch.nn.Linear):
     """``torch.nn.Linear`` with MLX's ``to_quantized`` hook, so that the
     reference's ``hasattr(module, "to_quantized")`` predicates select it."""

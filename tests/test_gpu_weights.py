@@ -94,3 +94,30 @@ def test_quantize_on_the_fly_then_save_and_reload(tmp_path, oracle, bits):
         for (ka, va), (kb, vb) in zip(model.state_dict().items(), fresh.state_dict().items()):
             assert ka == kb and vb.is_cuda and torch.equal(va.view(torch.uint8), vb.view(torch.uint8)), ka
         assert torch.equal(fresh(x), y1)
+
+
+@pytest.mark.parametrize("M", [1, 512, 4096])
+def test_concat_quantized_equals_the_separate_layers(M):
+    """q, k, v stacked along N give the three outputs side by side.  Each output
+    column depends on its own weight row only; the stacked shape may take a
+    different kernel or K cut, so sums can differ in their last float32 bits:
+    one bfloat16 ulp at the size of the row's largest output is allowed (the
+    bias is added after the product is rounded, so a small output can carry the
+    ulp of a larger product)."""
+    import mflux_amd
+    from mflux_amd import nn as qnn
+
+    torch.manual_seed(11)
+    K = 1024
+    layers = [qnn.QuantizedLinear.from_linear(torch.nn.Linear(K, n, bias=(n != 768), device="cuda", dtype=torch.bfloat16),
+                                              64, 4) for n in (1024, 768, 1024)]
+    fused = qnn.concat_quantized(layers)
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    y = fused(x)
+    parts = y.split([1024, 768, 1024], dim=-1)
+    for part, layer in zip(parts, layers):
+        ref = layer(x)
+        assert part.shape == ref.shape
+        bound = 2.0 ** -7 * ref.float().abs().amax(dim=-1, keepdim=True)
+        assert torch.all((part.float() - ref.float()).abs() <= bound)
+        assert (part != ref).float().mean() < 0.01   # and nearly all outputs are identical

@@ -172,6 +172,31 @@ def test_embedding_is_quantizable_and_walked():
     assert torch.equal(plain.as_linear(torch.ones(1, 64)), torch.ones(1, 64) @ plain.weight.T)
 
 
+def test_concat_quantized_stacks_rows_and_checks_compatibility():
+    a = qnn.QuantizedLinear(128, 64, bias=True, bits=4)
+    b = qnn.QuantizedLinear(128, 32, bias=False, bits=4)
+    c = qnn.QuantizedLinear(128, 16, bias=True, bits=4)
+    a.weight.fill_(1), b.weight.fill_(2), c.weight.fill_(3)
+    a.bias.fill_(0.5), c.bias.fill_(-1.0)
+    fused = qnn.concat_quantized([a, b, c])
+    assert isinstance(fused, qnn.QuantizedLinear) and (fused.input_dims, fused.output_dims) == (128, 112)
+    assert (fused.group_size, fused.bits, fused.mode) == (64, 4, "affine")
+    assert fused.weight.dtype == torch.uint32 and tuple(fused.weight.shape) == (112, 16)
+    assert tuple(fused.scales.shape) == (112, 2) and tuple(fused.biases.shape) == (112, 2)
+    assert fused.weight.view(torch.int32)[:, 0].tolist() == [1] * 64 + [2] * 32 + [3] * 16
+    assert fused.bias.tolist() == [0.5] * 64 + [0.0] * 32 + [-1.0] * 16     # a missing bias is zeros
+    assert sorted(fused.state_dict()) == ["bias", "biases", "scales", "weight"]
+    assert qnn.concat_quantized([b, b]).bias is None
+    with pytest.raises(ValueError, match="must share"):
+        qnn.concat_quantized([a, qnn.QuantizedLinear(128, 64, bits=8)])
+    with pytest.raises(ValueError, match="must share"):
+        qnn.concat_quantized([a, qnn.QuantizedLinear(256, 64, bits=4)])
+    with pytest.raises(ValueError, match="expected QuantizedLinear"):
+        qnn.concat_quantized([a, torch.nn.Linear(128, 64)])
+    with pytest.raises(ValueError, match="at least one"):
+        qnn.concat_quantized([])
+
+
 def test_quantized_linear_constructor_on_cpu_is_a_placeholder():
     q = qnn.QuantizedLinear(256, 64, bias=True, group_size=None, bits=8)
     assert (q.group_size, q.bits) == (64, 8)
