@@ -120,3 +120,61 @@ def _forward(owner: torch.nn.Module, base: torch.nn.Module, loras: list[LoRALine
     t = torch.matmul(x.to(compute), a_cat)
     return core.quantized_matmul(x, base.weight, base.scales, base.biases, transpose=True, group_size=base.group_size,
                                  bits=base.bits, mode=base.mode, bias=base.bias, low_rank=(t, bs))
+
+
+# ---- baking adapters into the base weights (for saving) -------------------------
+def _delta(lora: LoRALinear) -> torch.Tensor:
+    """``scale * (lora_A @ lora_B).T``, ``[out, in]``, in float32."""
+    return float(lora.scale) * torch.matmul(lora.lora_A.detach().float(), lora.lora_B.detach().float()).t()
+
+
+def _bake(base: torch.nn.Module, loras: list[LoRALinear], requantize: bool) -> None:
+    if not hasattr(base, "weight") or not loras:
+        return
+    quantized = isinstance(base, QuantizedLinear)
+    shape = (base.output_dims, base.input_dims) if quantized and requantize else tuple(base.weight.shape)
+    deltas = []
+    for lora in loras:
+        delta = _delta(lora)
+        if tuple(delta.shape) != shape:
+            print(f"⚠️  Skipping LoRA bake due to shape mismatch: weight {shape} vs delta {tuple(delta.shape)}")
+            continue
+        deltas.append(delta)
+    if not deltas:
+        return
+    if quantized:
+        # all adapters at once, so that the weight is requantized a single time
+        full = core.dequantize(base.weight, base.scales, base.biases, base.group_size, base.bits)
+        baked = (full.float() + sum(deltas).to(full.device)).to(full.dtype)
+        base.weight, base.scales, base.biases = core.quantize(baked, base.group_size, base.bits, base.mode)
+        return
+    with torch.no_grad():
+        for delta in deltas:   # one rounded add per adapter, as the reference does
+            base.weight.add_(delta.to(device=base.weight.device, dtype=base.weight.dtype))
+
+
+def bake_and_strip_lora(module: torch.nn.Module, requantize: bool = False) -> torch.nn.Module:
+    """Replaces every ``LoRALinear`` / ``FusedLoRALinear`` below ``module`` by its
+    base layer with the adapters added into the weight, as
+    ``LoRASaver.bake_and_strip_lora``
+    (src/mflux/models/common/lora/mapping/lora_saver.py:9-82) does before a
+    model is saved: ``weight += (scale * lora_A @ lora_B).T`` in the weight's
+    dtype.  Around a quantized base the reference's shapes do not match and it
+    strips the wrapper without baking (``:75-77``), and so does this function
+    by default; ``requantize=True`` instead dequantizes the base, adds the
+    adapters in float32, rounds to the 16-bit type and quantizes again with the
+    layer's group size and bits (lossy by one requantization).  Returns
+    ``module`` (the base layer when ``module`` itself is a wrapper)."""
+    def strip(obj: torch.nn.Module) -> torch.nn.Module:
+        if isinstance(obj, FusedLoRALinear):
+            _bake(obj.base_linear, [lora for lora in obj.loras if isinstance(lora, LoRALinear)], requantize)
+            return obj.base_linear
+        if isinstance(obj, LoRALinear):
+            _bake(obj.linear, [obj], requantize)
+            return obj.linear
+        return obj
+
+    module = strip(module)
+    for name, child in list(module.named_children()):
+        module._modules[name] = bake_and_strip_lora(child, requantize)
+    return module

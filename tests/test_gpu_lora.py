@@ -224,3 +224,40 @@ def test_lora_linear_on_plain_linear():
     x = torch.randn(10, 256, device="cuda").to(torch.bfloat16)
     with torch.no_grad():
         _assert_close(lora(x), _layer_ref(x, lin.weight, None, [lora]), tol=2e-2)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_bake_with_requantize_folds_the_adapters_into_the_codes(bits):
+    """requantize=True: the base's codes become quantize(dequantize(W) + delta);
+    the baked layer then answers like the wrapped one up to one requantization
+    (a quantization step of the weight, not the matmul tolerance)."""
+    import mflux_amd
+    from mflux_amd.lora import FusedLoRALinear, LoRALinear, bake_and_strip_lora
+
+    torch.manual_seed(6)
+    K, N, M = 512, 768, 300
+    lin = torch.nn.Linear(K, N, bias=True, device="cuda", dtype=torch.bfloat16)
+    q = mflux_amd.nn.QuantizedLinear.from_linear(lin, 64, bits)
+    loras = [LoRALinear.from_linear(q, r=8, scale=1.0), LoRALinear.from_linear(q, r=16, scale=-0.5)]
+    holder = torch.nn.Sequential(FusedLoRALinear(q, loras))
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    w_old = mflux_amd.dequantize(q.weight, q.scales, q.biases, 64, bits)
+    delta = sum(l.scale * (l.lora_A.float() @ l.lora_B.float()).t() for l in loras)
+    target = (w_old.float() + delta).to(torch.bfloat16)
+    with torch.no_grad():
+        wrapped = holder(x).double()
+    bake_and_strip_lora(holder, requantize=True)
+    assert holder[0] is q
+    wq, s, b = mflux_amd.quantize(target, 64, bits)
+    assert torch.equal(q.weight, wq) and torch.equal(q.scales, s) and torch.equal(q.biases, b)
+    w_new = mflux_amd.dequantize(q.weight, q.scales, q.biases, 64, bits).float()
+    step = q.scales.float().abs().repeat_interleave(64, dim=1)
+    # within one quantization step (the quantizer's own guarantee: it re-fits the scale to the group's
+    # edge, so the far end can be off by more than half a step), plus the rounding of the stored scale
+    # (times the code, up to 2^bits - 1) and of the dequantised value to bfloat16
+    slack = 1.0 + (2 ** bits - 1) * 2.0 ** -8
+    assert torch.all((w_new - target.float()).abs() <= slack * step + 2.0 ** -8 * target.float().abs() + 1e-6)
+    with torch.no_grad():
+        baked = q(x).double()
+    err = (baked - wrapped).abs().max() / wrapped.abs().max()
+    assert err < (0.15 if bits == 4 else 0.02)

@@ -346,3 +346,41 @@ def test_foreign_directory_is_not_our_format(tmp_path):
               metadata={"quantization_level": "None", "mflux_version": "0.1"})
     tree, level, version = W.try_load_saved_format(tmp_path / "hf")
     assert level is None and version == "0.1" and torch.equal(tree["w"], torch.zeros(2))
+
+
+def test_bake_and_strip_lora_on_float_and_quantized_bases(capsys):
+    """Wrappers are replaced by their bases wherever they sit in the tree; a
+    float base gets weight += (scale * A @ B).T; a quantized base is stripped
+    without baking, with the reference's warning (lora_saver.py:75-77)."""
+    from mflux_amd.lora import FusedLoRALinear, LoRALinear, bake_and_strip_lora
+
+    torch.manual_seed(0)
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.proj = LoRALinear.from_linear(torch.nn.Linear(32, 16, dtype=torch.float32), r=4, scale=0.5)
+            lin = torch.nn.Linear(32, 8, dtype=torch.float32)
+            self.heads = torch.nn.ModuleList([
+                FusedLoRALinear(lin, [LoRALinear.from_linear(lin, r=2, scale=1.0), LoRALinear.from_linear(lin, r=3, scale=-2.0)]),
+                torch.nn.Linear(8, 8),
+            ])
+            self.q = LoRALinear.from_linear(qnn.QuantizedLinear(64, 16, bias=False, bits=4), r=4)
+
+    net = Block()
+    x = torch.randn(5, 32)
+    want_proj, want_head = net.proj(x), net.heads[0](x)
+    w_before = net.heads[0].base_linear.weight.detach().clone()
+    loras = list(net.heads[0].loras)
+    packed_before = net.q.linear.weight.clone()
+    out = bake_and_strip_lora(net)
+    assert out is net
+    assert type(net.proj) is torch.nn.Linear and type(net.heads[0]) is torch.nn.Linear
+    assert isinstance(net.q, qnn.QuantizedLinear) and torch.equal(net.q.weight, packed_before)
+    assert "Skipping LoRA bake due to shape mismatch" in capsys.readouterr().out
+    delta = sum(l.scale * (l.lora_A.float() @ l.lora_B.float()).t() for l in loras)
+    assert torch.allclose(net.heads[0].weight, w_before + delta, atol=1e-6)
+    assert torch.allclose(net.proj(x), want_proj, atol=1e-5) and torch.allclose(net.heads[0](x), want_head, atol=1e-5)
+    # a wrapper passed in directly comes back as its baked base
+    top = LoRALinear.from_linear(torch.nn.Linear(8, 4, dtype=torch.float32), r=2)
+    assert type(bake_and_strip_lora(top)) is torch.nn.Linear
