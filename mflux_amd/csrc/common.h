@@ -173,6 +173,10 @@ int launch_dequantize_rows(const uint32_t* wq, const void* scales, const void* b
 int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream);
+// one activation row on the vector pipeline's integer dot product (qmv_dot_covers() says whether it takes a shape)
+bool qmv_dot_covers(int64_t M, int64_t K, int bits);
+int launch_qmv_dot(const void* x, int dtype, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                   const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream);
 // 3-, 5- and 6-bit weights, one activation row; MFQ_EUNSUPPORTED for shapes it does not take
 int launch_qmv_odd(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
