@@ -30,6 +30,8 @@
 // wavefronts in balanced contiguous runs.  The integer image of x is built by
 // the workgroup's four wavefronts together, through LDS, and then held in
 // registers.
+#include <type_traits>
+
 #include "common.h"
 
 namespace mfq {
@@ -156,7 +158,8 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
   extern __shared__ __attribute__((aligned(16))) uint32_t ximg[];  // [pieces][kXWords]
   __shared__ int wave_amax[4];
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  // uniform over the wavefront, and known to be: row addresses then live in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int row_bytes = K * BITS / 8;
   const int groups = K >> gs_shift;
 
@@ -266,6 +269,7 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
 
   if (row_begin >= row_end) return;  // behind the last barrier
 
+  uint32_t kept = 0;  // lane i: the finished output of the i-th row of the run in hand
   auto consume = [&](const R& regs, int64_t row) __attribute__((always_inline)) {
     float tot = 0.f;
 #pragma unroll
@@ -304,37 +308,61 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
       tot = __builtin_fmaf(sc, d, tot);
       tot = __builtin_fmaf(bo, sx[j], tot);
     }
+    // every lane holds the row's result; lane (row - row_begin) % 64 keeps it until flush()
     float v = wave_sum(tot) * unscale;
-    if (lane == 0) {
+    uint32_t out;
+    if (y_is_f32) {
+      if (bias) v += T::to_f32(regs.bias);
+      out = __builtin_bit_cast(uint32_t, v);
+    } else {
+      uint16_t hv = T::from_f32(v);
+      if (bias) hv = T::from_f32(T::to_f32(hv) + T::to_f32(regs.bias));
+      out = hv;
+    }
+    if (lane == (int)((row - row_begin) & 63)) kept = out;
+  };
+  // Stores the results of rows [first, first + count), count <= 64, one per lane.
+  // Results leave the wavefront once, at its end, and not row by row: a store
+  // in flight between the loads would make every wait for a load a wait for
+  // everything (loads and stores share one counter and may overtake each other).
+  auto flush = [&](int64_t first, int count) {
+    if (lane < count) {
       if (y_is_f32) {
-        if (bias) v += T::to_f32(regs.bias);
-        reinterpret_cast<float*>(y)[row] = v;
+        reinterpret_cast<uint32_t*>(y)[first + lane] = kept;
       } else {
-        uint16_t hv = T::from_f32(v);
-        if (bias) hv = T::from_f32(T::to_f32(hv) + T::to_f32(regs.bias));
-        reinterpret_cast<uint16_t*>(y)[row] = hv;
+        reinterpret_cast<uint16_t*>(y)[first + lane] = (uint16_t)kept;
       }
     }
   };
 
-  // kDepth rows in flight per wavefront: row r + kDepth - 1 is requested before row r is consumed
-#ifndef QMV_DOT_DEPTH
-#define QMV_DOT_DEPTH 2
-#endif
-  constexpr int kDepth = QMV_DOT_DEPTH;
-  static_assert(kDepth == 2, "the first row is requested during the set-up");
-  for (int64_t row = row_begin; row < row_end; row += kDepth) {
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-      const int64_t r = row + d;
-      if (r < row_end) {
-        if (r + kDepth - 1 < row_end)
-          regs[(d + kDepth - 1) % kDepth].issue(wbytes, scales, biases, bias, r + kDepth - 1, row_bytes, groups, piece,
-                                                grp, lane);
-        consume(regs[d], r);
-      }
+  // Two rows in flight per wavefront: row r + 1 is requested before row r is
+  // consumed.  Inside the loop nothing is conditional: behind a branch the
+  // compiler cannot know how many younger loads are in flight when it waits for
+  // row r, and waits for all of them.  So the loop takes rows in pairs, an odd
+  // run consumes its first row ahead of it (the loop then starts on the other
+  // register set), and the request past the run's last row re-reads that row
+  // (an L2 hit that is never consumed).
+  const int64_t last = row_end - 1;
+  auto pairs = [&](auto parity, int64_t first) __attribute__((always_inline)) {
+    constexpr int kP = decltype(parity)::value;  // register set that holds row `first`
+    for (int64_t row = first; row < row_end; row += 2) {
+      regs[kP ^ 1].issue(wbytes, scales, biases, bias, row + 1, row_bytes, groups, piece, grp, lane);
+      __builtin_amdgcn_sched_barrier(0);  // the requests stay in front of the arithmetic
+      consume(regs[kP], row);
+      regs[kP].issue(wbytes, scales, biases, bias, min(row + 2, last), row_bytes, groups, piece, grp, lane);
+      __builtin_amdgcn_sched_barrier(0);
+      consume(regs[kP ^ 1], row + 1);
     }
+  };
+  if ((row_end - row_begin) & 1) {
+    regs[1].issue(wbytes, scales, biases, bias, min(row_begin + 1, last), row_bytes, groups, piece, grp, lane);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(regs[0], row_begin);
+    pairs(std::integral_constant<int, 1>{}, row_begin + 1);
+  } else {
+    pairs(std::integral_constant<int, 0>{}, row_begin);
   }
+  flush(row_begin, (int)(row_end - row_begin));  // at most 64 rows per wavefront (the launcher sees to it)
 }
 
 template <typename T, int BITS, int kLoads, bool kCoop>
@@ -351,6 +379,8 @@ int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scal
   int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
   const int64_t max_blocks = (N + 3) / 4;  // at least one row per wavefront
   if (blocks > max_blocks) blocks = max_blocks;
+  const int64_t min_blocks = (N + 255) / 256;  // at most 64 rows per wavefront: a lane keeps one result
+  if (blocks < min_blocks) blocks = min_blocks;
   const int64_t n_waves = blocks * 4;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), lds, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
