@@ -6,7 +6,9 @@
 // one or a few activation rows against a wide weight, so the kernel is bound
 // by streaming the packed weight from HBM once.
 //
-// Two kernels here; a third, for two to four activation rows, is in
+// Two kernels here.  One activation row against rows of up to 6 KiB (W8) or
+// 3 KiB (W4) of codes, which is every such call mflux makes, runs the integer
+// dot-product kernel of qmv_dot.hip; two to four activation rows the kernel of
 // qmv_quad.hip.
 //
 // qmv_rows_kernel (M <= 4, rows of at most 6 KiB of codes): one wavefront per

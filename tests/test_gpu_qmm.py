@@ -176,6 +176,71 @@ def test_qmv_one_hot_and_float32_output(oracle):
             assert np.all(np.abs(got - deq[:, k]) <= 2.0 ** -8 * np.abs(deq[:, k]) + 1e-3 * step[:, k // 64]), (bits, k)
 
 
+def _one_row_ref(o, x_bits, wq, s, b, bits, gs=64):
+    xf = o.bf16_bits_to_f32(x_bits).astype(np.float64)
+    return o.quantized_matmul_f64(xf, wq, s, b, o.BF16, gs, bits)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_qmv_one_row_fixed_point_image_of_x(oracle, bits):
+    """The one-row kernel turns x into 15-bit fixed point with one power-of-two
+    scale per row.  Small integers stay exact (float32 output reproduces the
+    integer result bit for bit); a row whose elements span many orders of
+    magnitude loses at most 2^-15 of its largest element per element; tiny and
+    huge rows are rescaled without under- or overflow; a zero row gives the
+    bias; an infinity in x makes every output NaN."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    rng = np.random.default_rng(31 + bits)
+    K, N = 3072, 520
+    n_bins = 2 ** bits - 1
+    codes = rng.integers(0, n_bins + 1, (N, K)).astype(np.float32)
+    codes[:, ::64] = 0
+    codes[:, 1::64] = n_bins          # every group spans 0..n_bins: scale 1 (or -1), dequantised weight = code
+    w_bits = o.f32_to_bf16_bits(codes)
+    wq, s, b = o.c_quantize(w_bits, o.BF16, 64, bits)
+    assert np.array_equal(o.dequantize_exact(wq, s, b, o.BF16, 64, bits), codes)
+    dev = lambda a: to_dev(a, o.BF16)
+    run = lambda xb, **kw: mflux_amd.quantized_matmul(dev(xb).float(), u32_to_dev(wq), dev(s), dev(b), group_size=64,
+                                                      bits=bits, **kw).cpu().numpy().astype(np.float64)
+    # small integers: exact
+    xi = rng.integers(-3, 4, (1, K)).astype(np.float32)
+    assert np.array_equal(run(o.f32_to_bf16_bits(xi)), xi.astype(np.float64) @ codes.astype(np.float64).T)
+    # a wide dynamic range: bound from the rounding of x alone, plus float32 rounding of the sums
+    xw = (rng.standard_normal((1, K)) * 10.0 ** rng.integers(-6, 3, (1, K))).astype(np.float32)
+    xb = o.f32_to_bf16_bits(xw)
+    xmax = np.abs(o.bf16_bits_to_f32(xb)).max()
+    ref = _one_row_ref(o, xb, wq, s, b, bits)
+    bound = 2.0 ** -15 * xmax * np.abs(codes).sum(axis=1) + 2.0 ** -20 * np.abs(ref)
+    assert np.all(np.abs(run(xb) - ref) <= bound)
+    # tiny and huge rows (the scale's exponent is clamped for the former), against float64
+    for mag in (1e-30, 1e-12, 1e20, 1e30):
+        xb = o.f32_to_bf16_bits((rng.standard_normal((1, K)) * mag).astype(np.float32))
+        ref = _one_row_ref(o, xb, wq, s, b, bits)
+        got = run(xb)
+        assert np.all(np.isfinite(got)) and np.all(np.abs(got - ref) <= 1e-3 * np.abs(ref).max())
+    # zeros give the bias exactly; an infinity anywhere gives NaN everywhere
+    bias = o.f32_to_bf16_bits(seeded(32, 2, (N,), 1.0))
+    zero = np.zeros((1, K), dtype=np.uint16)
+    assert np.array_equal(run(zero, bias=dev(bias))[0], o.bf16_bits_to_f32(bias).astype(np.float64))
+    xinf = o.f32_to_bf16_bits(xi.copy())
+    xinf[0, 1000] = 0x7f80
+    assert np.all(np.isnan(run(xinf)))
+
+
+@pytest.mark.parametrize("N", [1, 2, 3, 5, 63, 262144 + 8])
+def test_qmv_one_row_run_lengths(oracle, N):
+    """Rows are dealt to wavefronts in runs of up to 64 (a lane keeps one
+    result until the run ends): fewer rows than wavefronts in a workgroup, odd
+    and even runs, and runs of the full 64 rows."""
+    o = oracle
+    K = 64
+    args = _case(o, 33, 1, K, N, 8, with_bias=True)
+    _assert_close(_run(o, *args, 8), _ref(o, *args, 8))
+
+
 def test_qmv_adaln_config_full(oracle):
     """The adaLN modulation shape: SiLU(temb) [M,3072] against W8 [18432,3072]."""
     o = oracle
