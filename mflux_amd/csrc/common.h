@@ -183,7 +183,7 @@ int launch_qmv_odd(const void* x, int dtype, int64_t M, int64_t K, const uint32_
                    hipStream_t stream);
 // four weight rows at a time, M <= 4 (qmv_quad_covers() says whether it takes a shape)
 bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* scales, const void* biases,
-                     const void* y, int y_dtype);
+                     const void* bias, const void* y, int y_dtype);
 int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                     hipStream_t stream);

@@ -592,7 +592,7 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
     return launch_qmv_dot(x, dtype, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   // two to four activation rows: four weight rows at a time (for a single row
   // the one-row-per-wavefront kernel below is the faster of the two)
-  if (M >= 2 && qmv_quad_covers(M, K, N, gs, bits, scales, biases, y, y_dtype))
+  if (M >= 2 && qmv_quad_covers(M, K, N, gs, bits, scales, biases, bias, y, y_dtype))
     return launch_qmv_quad(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   if (rows_kernel_covers(M, K, bits)) {
     if (dtype == MFQ_BF16)

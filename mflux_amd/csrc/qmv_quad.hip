@@ -73,7 +73,8 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   extern __shared__ __attribute__((aligned(16))) char lds[];  // x operands, slice sums, 4 x 2 scale regions
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
+  // uniform over the wavefront, and known to be: quad addresses then live in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int blk = lane >> 2, li = lane & 3;
   const int row_bytes = kLoads * 256;
   const int groups = K >> gs_shift;
@@ -93,7 +94,9 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   const int quad_sb_bytes = 8 * groups;  // four rows of one array
   const char* sb_src = reinterpret_cast<const char*>(lane < 32 ? scales : biases);
   const int sb_off = (lane & 31) * 16;
-  const bool sb_lane = sb_off < quad_sb_bytes;
+  // lanes past the quad's block re-read its last 16 bytes (into a part of the region nobody reads): a
+  // load behind a branch would make the number of loads in flight unknown to the waits that follow
+  const int sb_off_load = min(sb_off, quad_sb_bytes - 16);
   // where this lane finds the scale of piece (j, blk) of row li inside a region
   const int piece_groups = (16 * kCodes) >> gs_shift;  // groups one load instruction spans
   const int sidx0 = (li * groups + ((blk * kCodes) >> gs_shift)) * 2;
@@ -103,9 +106,7 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   asm volatile("" : "+s"(pair_mask), "+v"(magic), "+v"(magic_high));
 
   auto load_scales = [&](int q) __attribute__((always_inline)) {
-    u32x4 v = {0, 0, 0, 0};
-    if (sb_lane) v = *reinterpret_cast<const u32x4*>(sb_src + (size_t)q * quad_sb_bytes + sb_off);
-    return v;
+    return *reinterpret_cast<const u32x4*>(sb_src + (size_t)q * quad_sb_bytes + sb_off_load);
   };
   auto store_scales = [&](u32x4 v, int buf) __attribute__((always_inline)) {
     *reinterpret_cast<u32x4*>(sreg + buf * kScaleRegion + (lane >> 5) * 512 + sb_off) = v;
@@ -165,6 +166,13 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   for (int q = q_begin; q < q_end; ++q) {
     const int qn = min(q + 1, q_end - 1);  // past the end: this wavefront's last quad again, never consumed
     const u32x4 sb_next = load_scales(qn);
+    // the quad's four bias values, requested now and unconditionally (without a bias: from the scales,
+    // unused): fetched where they are needed, behind a branch, the wait for them would have to cover
+    // every weight load in flight and drain the ring once per quad
+    // The address is uniform and 8-byte aligned (the launcher checks), which makes this a scalar load
+    // with a counter of its own.
+    const uint2 bq2 = static_cast<const uint2*>(__builtin_assume_aligned(bias ? bias : scales, 8))[q];
+    const uint16_t bq[4] = {(uint16_t)bq2.x, (uint16_t)(bq2.x >> 16), (uint16_t)bq2.y, (uint16_t)(bq2.y >> 16)};
     const char* sb = sreg + (q & 1) * kScaleRegion + sidx0;
     f32x4 tot = {0.f, 0.f, 0.f, 0.f};  // register i: row r0+i against this lane's activation row
     for_each_index<kLoads>([&](auto jc) __attribute__((always_inline)) {
@@ -239,7 +247,7 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
       float bv[4] = {0.f, 0.f, 0.f, 0.f};
       if (bias) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bv[i] = T::to_f32(bias[r0 + i]);
+        for (int i = 0; i < 4; ++i) bv[i] = T::to_f32(bq[i]);
       }
       const int64_t o = (int64_t)lane * N + r0;
       if (y_is_f32) {
@@ -319,7 +327,8 @@ int launch_loads(int64_t loads, const void* x, int64_t M, int64_t K, const uint3
 // bytes); K <= 4096 (the x operands' LDS copy); pointers aligned for the
 // 16-byte scale fetches and the 8- / 16-byte stores.
 bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* scales, const void* biases,
-                     const void* y, int y_dtype) {
+                     const void* bias, const void* y, int y_dtype) {
+  if (reinterpret_cast<uintptr_t>(bias) & 7u) return false;  // four bias values travel as one 8-byte load
   const int64_t row_bytes = K * bits / 8;
   const int64_t loads = row_bytes / 256;
   const int64_t groups = K / gs;
