@@ -309,17 +309,14 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
       tot = __builtin_fmaf(bo, sx[j], tot);
     }
     // every lane holds the row's result; lane (row - row_begin) % 64 keeps it until flush()
-    float v = wave_sum(tot) * unscale;
-    uint32_t out;
-    if (y_is_f32) {
-      if (bias) v += T::to_f32(regs.bias);
-      out = __builtin_bit_cast(uint32_t, v);
-    } else {
-      uint16_t hv = T::from_f32(v);
-      if (bias) hv = T::from_f32(T::to_f32(hv) + T::to_f32(regs.bias));
-      out = hv;
-    }
-    if (lane == (int)((row - row_begin) & 63)) kept = out;
+    // (selects, not branches: the loop body stays one block, which keeps the requests where they are put)
+    const float v = wave_sum(tot) * unscale;
+    const float bv = T::to_f32(regs.bias);
+    const float v32 = bias ? v + bv : v;
+    const uint16_t h0 = T::from_f32(v);
+    const uint16_t h1 = T::from_f32(T::to_f32(h0) + bv);  // second rounding, as a separate add on the 16-bit result
+    const uint32_t out = y_is_f32 ? __builtin_bit_cast(uint32_t, v32) : (uint32_t)(bias ? h1 : h0);
+    kept = lane == (int)((row - row_begin) & 63) ? out : kept;
   };
   // Stores the results of rows [first, first + count), count <= 64, one per lane.
   // Results leave the wavefront once, at its end, and not row by row: a store
@@ -346,9 +343,12 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
   auto pairs = [&](auto parity, int64_t first) __attribute__((always_inline)) {
     constexpr int kP = decltype(parity)::value;  // register set that holds row `first`
     for (int64_t row = first; row < row_end; row += 2) {
+      // the requests stay between the arithmetic of two rows, in front of the waits for the older row
+      __builtin_amdgcn_sched_barrier(0);
       regs[kP ^ 1].issue(wbytes, scales, biases, bias, row + 1, row_bytes, groups, piece, grp, lane);
-      __builtin_amdgcn_sched_barrier(0);  // the requests stay in front of the arithmetic
+      __builtin_amdgcn_sched_barrier(0);
       consume(regs[kP], row);
+      __builtin_amdgcn_sched_barrier(0);
       regs[kP].issue(wbytes, scales, biases, bias, min(row + 2, last), row_bytes, groups, piece, grp, lane);
       __builtin_amdgcn_sched_barrier(0);
       consume(regs[kP ^ 1], row + 1);

@@ -101,7 +101,8 @@ __global__ __launch_bounds__(256) void qmv_odd_kernel(const uint16_t* __restrict
   }
 
   // rows are dealt to wavefronts in contiguous, balanced runs (split computed on the host)
-  const int wave_id = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  // (the wavefront index read as a scalar: row addresses then live in scalar registers)
+  const int wave_id = blockIdx.x * (blockDim.x / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t row_begin = (int64_t)wave_id * rows_per_wave + min(wave_id, extra_rows);
   const int64_t row_end = row_begin + rows_per_wave + (wave_id < extra_rows ? 1 : 0);
   if (row_begin >= row_end) return;
@@ -134,9 +135,10 @@ __global__ __launch_bounds__(256) void qmv_odd_kernel(const uint16_t* __restrict
 #pragma unroll
       for (int e = 0; e < BITS; ++e) r.w[j][e] = u.d[e];
     }
-    r.bias = bias ? bias[row] : (uint16_t)0;
+    r.bias = (bias ? bias + row : srow)[0];  // without a bias: any readable address, the value is not used
   };
 
+  uint32_t kept = 0;  // lane i: the finished output of the i-th row of the wavefront's run
   auto consume = [&](const Row& r, int64_t row) __attribute__((always_inline)) {
     f32x4 tot = {0.f, 0.f, 0.f, 0.f};  // register lane%4: this lane's sum of scale * D over its units
     float corr = 0.f;                  // this lane's sum of (bias - offset * scale) * sum(x)
@@ -174,28 +176,59 @@ __global__ __launch_bounds__(256) void qmv_odd_kernel(const uint16_t* __restrict
     }
     const int diag = lane & 3;
     float v = (diag == 0 ? tot[0] : diag == 1 ? tot[1] : diag == 2 ? tot[2] : tot[3]) + corr;
-    v = wave_sum(v);
-    if (lane == 0) {
-      if (y_is_f32) {
-        if (bias) v += T::to_f32(r.bias);
-        reinterpret_cast<float*>(y)[row] = v;
-      } else {
-        uint16_t hv = T::from_f32(v);
-        if (bias) hv = T::from_f32(T::to_f32(hv) + T::to_f32(r.bias));
-        reinterpret_cast<uint16_t*>(y)[row] = hv;
-      }
-    }
+    v = wave_sum(v);  // in every lane; lane (row - row_begin) % 64 keeps the row's output until the run ends
+    // (selects, not branches: the loop body stays one block, which keeps the requests where they are put)
+    const float bv = T::to_f32(r.bias);
+    const float v32 = bias ? v + bv : v;
+    const uint16_t h0 = T::from_f32(v);
+    const uint16_t h1 = T::from_f32(T::to_f32(h0) + bv);  // second rounding, as a separate add on the 16-bit result
+    const uint32_t out = y_is_f32 ? __builtin_bit_cast(uint32_t, v32) : (uint32_t)(bias ? h1 : h0);
+    kept = lane == (int)((row - row_begin) & 63) ? out : kept;
   };
 
-  // two rows in flight per wavefront: row r + 1 is requested before row r is consumed
-  Row ra, rb;
-  issue(ra, row_begin);
-  for (int64_t row = row_begin; row < row_end; row += 2) {
-    if (row + 1 < row_end) issue(rb, row + 1);
-    consume(ra, row);
-    if (row + 1 < row_end) {
-      if (row + 2 < row_end) issue(ra, row + 2);
-      consume(rb, row + 1);
+  // Two rows in flight per wavefront: row r + 1 is requested before row r is
+  // consumed.  Inside the loop nothing is conditional and nothing is stored:
+  // behind a branch the compiler cannot know how many younger loads are in
+  // flight when it waits for row r, and waits for all of them (a store between
+  // the loads has the same effect).  So the loop takes rows in pairs, an odd run
+  // consumes its first row ahead of it (the loop then starts on the other
+  // register set), the request past the run's last row re-reads that row, and
+  // the run's outputs (at most 64, the launcher sees to it) leave together.
+  Row rr[2];
+  issue(rr[0], row_begin);
+  const int64_t last = row_end - 1;
+  auto fence = [] () __attribute__((always_inline)) {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto pairs = [&](auto parity, int64_t first) __attribute__((always_inline)) {
+    constexpr int kP = decltype(parity)::value;  // register set that holds row `first`
+    for (int64_t row = first; row < row_end; row += 2) {
+      // the requests stay between the arithmetic of two rows, in front of the waits for the older row
+      // (the empty asm keeps the optimiser, the scheduling barrier the scheduler from moving them)
+      fence();
+      issue(rr[kP ^ 1], row + 1);
+      fence();
+      consume(rr[kP], row);
+      fence();
+      issue(rr[kP], min(row + 2, last));
+      fence();
+      consume(rr[kP ^ 1], row + 1);
+    }
+  };
+  if ((row_end - row_begin) & 1) {
+    issue(rr[1], min(row_begin + 1, last));
+    fence();
+    consume(rr[0], row_begin);
+    pairs(std::integral_constant<int, 1>{}, row_begin + 1);
+  } else {
+    pairs(std::integral_constant<int, 0>{}, row_begin);
+  }
+  if (lane < (int)(row_end - row_begin)) {
+    if (y_is_f32) {
+      reinterpret_cast<uint32_t*>(y)[row_begin + lane] = kept;
+    } else {
+      reinterpret_cast<uint16_t*>(y)[row_begin + lane] = (uint16_t)kept;
     }
   }
 }
@@ -214,6 +247,8 @@ int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scal
   int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
   const int64_t max_blocks = (N + 3) / 4;
   if (blocks > max_blocks) blocks = max_blocks;
+  const int64_t min_blocks = (N + 255) / 256;  // at most 64 rows per wavefront: a lane keeps one result
+  if (blocks < min_blocks) blocks = min_blocks;
   const int64_t n_waves = blocks * 4;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
