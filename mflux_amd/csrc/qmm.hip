@@ -39,7 +39,8 @@ constexpr int kThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;   // one 16-bit x tile: 32 KiB
 constexpr int kStageStride = 144;         // bytes per staged output row: 64 16-bit columns + 16 bytes of padding
 constexpr int kStageBytes = 128 * kStageStride;  // one wavefront stages 128 rows of its 64 columns at a time
-constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes;  // double-buffered x tiles + output staging
+constexpr int kBiasBytes = 64 * 4;  // per wavefront: the bias of its 64 columns as float32
+constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes + 4 * kBiasBytes;  // x tiles (double-buffered) + output staging + bias
 constexpr int kWriteSub = 2;  // sub-step whose fillers publish the next x tile to LDS
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -545,6 +546,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int lane = lane_e;
     char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
     uint16_t* yout = reinterpret_cast<uint16_t*>(out_base);
+    // the bias of the wavefront's 64 columns: one load (lane l takes column l), parked in LDS as
+    // float32 and read back four columns at a time; fetched value by value where it is used, every
+    // fetch would be waited for on its own, 32 times per tile
+    const float* bias_f = reinterpret_cast<const float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes);
+    if constexpr (kBias) {
+      *reinterpret_cast<float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes + lane * 4) =
+          T::to_f32(out_bias[min(n0 + wn + lane, N - 1)]);
+    }
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
@@ -554,8 +563,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           const int cl = 32 * j + 8 * eb + 4 * h;  // column inside the wavefront's 64
           float bv[4] = {0.f, 0.f, 0.f, 0.f};
           if constexpr (kBias) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(out_bias[min(n0 + wn + cl + c, N - 1)]);
+            const float4 b4 = *reinterpret_cast<const float4*>(bias_f + cl);
+            bv[0] = b4.x, bv[1] = b4.y, bv[2] = b4.z, bv[3] = b4.w;
           }
 #pragma unroll
           for (int a4 = 0; a4 < 4; ++a4) {
