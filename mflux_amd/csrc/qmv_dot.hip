@@ -370,13 +370,26 @@ int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scal
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
   auto kernel = qmv_dot_kernel<T, BITS, kLoads, kCoop>;
   const size_t lds = (size_t)(K * BITS / 8 / 16) * (BITS == 8 ? 8 : 16) * 4;  // the x image: 2 bytes per element
-  static int blocks_per_cu = 0;
-  if (blocks_per_cu == 0) {
+  static int resident = 0;  // workgroups of this instantiation a compute unit holds
+  if (resident == 0) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, lds) != hipSuccess || n < 1) n = 1;
-    blocks_per_cu = n > 4 ? 4 : n;
+    resident = n > 4 ? 4 : n;
   }
-  int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
+  // Workgroups per compute unit: enough wavefronts for about 48 KiB of weight rows in flight (two
+  // rows each), not more: every workgroup pays for its own image of x.  Measured at K = 3072: two
+  // workgroups for 3 KiB rows (W8), four for 1.5 KiB rows (W4).  One fewer when that deals the rows
+  // out evenly and the count in hand does not (18432 rows: 6 each on 3072 wavefronts, 4.5 on 4096).
+  const int64_t row_bytes = K * BITS / 8;
+  int per_cu = (int)((48 * 1024 / (2 * row_bytes) + 3) / 4);
+  per_cu = per_cu < 2 ? 2 : per_cu > 4 ? 4 : per_cu;
+  auto uneven = [&](int b) {
+    const int64_t waves = (int64_t)compute_units() * b * 4;
+    return N % waves != 0 && N > waves;
+  };
+  if (per_cu > 2 && uneven(per_cu) && !uneven(per_cu - 1)) --per_cu;
+  if (per_cu > resident) per_cu = resident;
+  int64_t blocks = (int64_t)compute_units() * per_cu;
   const int64_t max_blocks = (N + 3) / 4;  // at least one row per wavefront
   if (blocks > max_blocks) blocks = max_blocks;
   const int64_t min_blocks = (N + 255) / 256;  // at most 64 rows per wavefront: a lane keeps one result
