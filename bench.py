@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # plain copy of known size; the figures and the commands are in
 # profiles/qmm_w4a16_flux_single_block_m4608.md.  Not measurable from inside
 # this script.
-TRAFFIC_BYTES_PER_LAUNCH = ((556.9e6 + 202.6e6) + (503.0e6 + 32.1e6)) / 2
+TRAFFIC_BYTES_PER_LAUNCH = ((561.9e6 + 208.8e6) + (503.6e6 + 33.0e6)) / 2
 
 M_TOKENS = 4608
 LINEARS = (("linear1", 3072, 21504), ("linear2", 15360, 3072))  # (name, K, N)
