@@ -281,11 +281,13 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
       return MFQ_ELAUNCH;
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, kLds) != hipSuccess || n < 1) n = 1;
-    blocks_per_cu = n > 4 ? 4 : n;
+    // two workgroups per compute unit: every workgroup stages x for itself, and more of them measured
+    // slower (3072 -> 18432 at M = 4: 17.8 us with two, 19.0 us with three or four)
+    blocks_per_cu = n > 2 ? 2 : n;
   }
-  // At most as many wavefronts as are resident at once, and every one of them
-  // the same number of quads: with 4608 quads, 2304 wavefronts of two finish
-  // together, whereas 4096 wavefronts would leave 512 of them a second quad.
+  // At most that many wavefronts, and every one of them the same number of
+  // quads: with 4608 quads, 1536 wavefronts of three finish together, whereas
+  // 2048 wavefronts would leave 512 of them a third quad.
   const int64_t quads = N / 4;
   const int64_t max_waves = (int64_t)compute_units() * blocks_per_cu * 4;
   const int64_t per_wave = (quads + max_waves - 1) / max_waves;
