@@ -297,6 +297,23 @@ def main():
             res[f"M{Mg}"] = {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
                              "bytes": nbytes,
                              "weights": f"rotating over {n_buf} buffers ({n_buf * Ng * Kg * bits_g // 8 >> 20} MiB)"}
+        # the whole modulation call linear(silu(temb)) at M = 1: the activation inside the matvec
+        # kernel against an elementwise pass in front of it (what the reference runs)
+        temb16 = torch.randn(1, Kg, device=dev, generator=gen).to(torch.bfloat16)
+        state = {"i": 0}
+
+        def fused_call():
+            wqg, sg, bg = bufs[state["i"] % n_buf]
+            state["i"] += 1
+            mflux_amd.silu_quantized_matmul(temb16, wqg, sg, bg, group_size=GS, bits=bits_g, bias=bias)
+
+        def separate_call():
+            wqg, sg, bg = bufs[state["i"] % n_buf]
+            state["i"] += 1
+            mflux_amd.quantized_matmul(mflux_amd.silu(temb16), wqg, sg, bg, group_size=GS, bits=bits_g, bias=bias)
+
+        res["M1_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
+                               "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
         gemv[f"w{bits_g}"] = res
         del bufs
 

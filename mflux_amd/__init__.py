@@ -3,7 +3,8 @@ linears, a drop-in for the MLX operations mflux's diffusion transformers run
 through (``mx.quantize`` / ``nn.quantize`` / ``QuantizedLinear`` /
 ``mx.quantized_matmul``)."""
 from . import lora, nn, weights
-from .core import dequantize, dequantize_rows, quantize, quantized_matmul
+from .core import dequantize, dequantize_rows, quantize, quantized_matmul, silu, silu_quantized_matmul
 
-__all__ = ["nn", "lora", "weights", "quantize", "dequantize", "dequantize_rows", "quantized_matmul"]
+__all__ = ["nn", "lora", "weights", "quantize", "dequantize", "dequantize_rows", "quantized_matmul", "silu",
+           "silu_quantized_matmul"]
 __version__ = "0.1.0"

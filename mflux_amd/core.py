@@ -242,6 +242,59 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
     return _quantized_matmul_forward(x, w, scales, biases, group_size, bits, bias, low_rank)
 
 
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """``x * sigmoid(x)`` as MLX's ``nn.silu`` evaluates it: two operations in
+    ``x``'s dtype, so on a 16-bit tensor the sigmoid is rounded before the
+    product is (``torch.nn.functional.silu`` rounds once)."""
+    return x * torch.sigmoid(x)
+
+
+def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+                          group_size: int = 64, bits: int = 4, mode: str = "affine", *,
+                          bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``quantized_matmul(silu(x), w, scales, biases, transpose=True) (+ bias)``: the
+    adaLN modulation call ``self.linear(nn.silu(text_embeddings))`` of
+    src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 (and
+    ada_layer_norm_zero_single.py:12, ada_layer_norm_continuous.py:15).
+
+    For one row of 16-bit ``x`` against 4- or 8-bit weights the activation runs
+    inside the matvec kernel, where the row is converted anyway
+    (``mfq_qmv_silu``); for any other call it is :func:`silu`, an elementwise
+    pass, in front of :func:`quantized_matmul`.  Both round the sigmoid and the
+    product to ``x``'s dtype.  Not differentiable in its fused form: with
+    gradients enabled on ``x`` or ``bias`` the composed form runs.
+    """
+    _check_mode("quantized_matmul", mode)
+    _check_group_bits("quantized_matmul", group_size, bits)
+    needs_grad = torch.is_grad_enabled() and (x.requires_grad or (bias is not None and bias.requires_grad))
+    K = w.shape[-1] * 32 // bits
+    one_row = x.ndim >= 1 and x.shape[-1] == K and x.numel() == K
+    fusable = (one_row and not needs_grad and w.ndim == 2 and bits in MATMUL_KERNEL_BITS
+               and x.dtype == scales.dtype and x.dtype in (torch.bfloat16, torch.float16))
+    if fusable:
+        _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
+        _require_hip("quantized_matmul", x, "x")
+        _require_hip("quantized_matmul", w, "w")
+        N = w.shape[0]
+        if bias is not None:
+            if bias.shape != (N,):
+                raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
+            bias = bias.to(x.dtype).contiguous()
+        x1 = x.reshape(K).contiguous()
+        w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+        y = torch.empty((1, N), dtype=x.dtype, device=x.device)
+        with torch.cuda.device(x.device):
+            rc = _lib.load().mfq_qmv_silu(
+                x1.data_ptr(), _DTYPE_CODE[x.dtype], K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+                _DTYPE_CODE[x.dtype], bias.data_ptr() if bias is not None else None, N, group_size, bits,
+                y.data_ptr(), _DTYPE_CODE[x.dtype], _stream_ptr(x.device))
+        if rc != _lib.MFQ_EUNSUPPORTED:
+            _lib.check("mfq_qmv_silu", rc)
+            return y.reshape(*x.shape[:-1], N)
+    return quantized_matmul(silu(x), w, scales, biases, transpose=True, group_size=group_size, bits=bits, mode=mode,
+                            bias=bias)
+
 def _low_rank_operands(low_rank, lead: tuple, M: int, N: int, compute: torch.dtype):
     """Checks ``(t, bs)`` against the product's shape; returns them as contiguous
     ``[M, R]`` / ``[N, R]`` matrices in the compute dtype."""

@@ -175,8 +175,10 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                hipStream_t stream);
 // one activation row on the vector pipeline's integer dot product (qmv_dot_covers() says whether it takes a shape)
 bool qmv_dot_covers(int64_t M, int64_t K, int bits);
+// `silu`: the row that meets the weights is silu(x), each value rounded to `dtype`
 int launch_qmv_dot(const void* x, int dtype, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                   const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream);
+                   const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream,
+                   bool silu = false);
 // 3-, 5- and 6-bit weights, one activation row; MFQ_EUNSUPPORTED for shapes it does not take
 int launch_qmv_odd(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,

@@ -112,6 +112,25 @@ __device__ inline void split4(uint32_t p0, uint32_t p1, float mult, uint32_t& hi
   }
 }
 
+// SiLU of a pair of 16-bit floats as MLX's nn.silu computes it on that type,
+// x * sigmoid(x) with the sigmoid rounded to the type before the product
+// (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 feeds
+// nn.silu(text_embeddings) to the modulation linear).
+template <typename T>
+__device__ inline uint32_t silu_pair(uint32_t pair) {
+  uint32_t out = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float v = h ? hi_f32<T>(pair) : lo_f32<T>(pair);
+    // hardware exponential and reciprocal (one ulp each, far inside the rounding to 16 bits that follows);
+    // a denormal exponential flushed to 0 leaves the sigmoid at 1, an overflowing one makes it 0
+    const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
+    const float sg = T::to_f32(T::from_f32(__builtin_amdgcn_rcpf(1.f + e)));
+    out |= (uint32_t)T::from_f32(v * sg) << (16 * h);
+  }
+  return out;
+}
+
 template <typename T, int BITS, int kLoads, bool kCoop>
 struct DotRow {
   u32x4 w[kLoads];
@@ -145,7 +164,7 @@ struct DotRow {
   }
 };
 
-template <typename T, int BITS, int kLoads, bool kCoop>
+template <typename T, int BITS, int kLoads, bool kCoop, bool kSilu>
 __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq,
                                                       const uint16_t* __restrict__ scales,
                                                       const uint16_t* __restrict__ biases,
@@ -202,6 +221,14 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
   // (a wavefront without rows, which a grid rounded up to whole workgroups can leave, re-reads the last row)
   regs[0].issue(wbytes, scales, biases, bias, min(row_begin, (int64_t)N - 1), row_bytes, groups, piece, grp, lane);
 
+  if constexpr (kSilu) {  // the activation in front of the linear, on the values as they arrive
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      if (wave * kWave + 256 * i >= n_chunks) continue;  // a wavefront whose chunks all lie past the end
+#pragma unroll
+      for (int q = 0; q < kRawWords; ++q) raw[i][q] = silu_pair<T>(raw[i][q]);
+    }
+  }
   int amax = 0;
 #pragma unroll
   for (int i = 0; i < kLoads; ++i)
@@ -365,10 +392,10 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
   flush(row_begin, (int)(row_end - row_begin));  // at most 64 rows per wavefront (the launcher sees to it)
 }
 
-template <typename T, int BITS, int kLoads, bool kCoop>
+template <typename T, int BITS, int kLoads, bool kCoop, bool kSilu>
 int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
-  auto kernel = qmv_dot_kernel<T, BITS, kLoads, kCoop>;
+  auto kernel = qmv_dot_kernel<T, BITS, kLoads, kCoop, kSilu>;
   const size_t lds = (size_t)(K * BITS / 8 / 16) * (BITS == 8 ? 8 : 16) * 4;  // the x image: 2 bytes per element
   static int resident = 0;  // workgroups of this instantiation a compute unit holds
   if (resident == 0) {
@@ -401,18 +428,20 @@ int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scal
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
-template <typename T, int BITS, int kLoads>
+template <typename T, int BITS, int kLoads, bool kSilu>
 int launch_loads(int64_t n_loads, const void* x, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                  const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
   if (n_loads == kLoads) {
     const int64_t groups = K >> gs_shift;
     const bool coop = groups <= 64 && groups % 2 == 0 &&
                       ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 3u) == 0;
-    if (coop) return launch_kernel<T, BITS, kLoads, true>(x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-    return launch_kernel<T, BITS, kLoads, false>(x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    if (coop)
+      return launch_kernel<T, BITS, kLoads, true, kSilu>(x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    return launch_kernel<T, BITS, kLoads, false, kSilu>(x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
   }
   if constexpr (kLoads > 1)
-    return launch_loads<T, BITS, kLoads - 1>(n_loads, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    return launch_loads<T, BITS, kLoads - 1, kSilu>(n_loads, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype,
+                                                    stream);
   return MFQ_EUNSUPPORTED;
 }
 
@@ -421,14 +450,14 @@ int launch_loads(int64_t n_loads, const void* x, int64_t K, const uint32_t* wq, 
 constexpr int kMaxLoadsW8 = 6;
 constexpr int kMaxLoadsW4 = 3;
 
-template <typename T>
+template <typename T, bool kSilu>
 int launch_type(const void* x, int64_t K, const uint32_t* wq, const void* scales, const void* biases, const void* bias,
                 int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream) {
   const int gs_shift = gs == 32 ? 5 : gs == 64 ? 6 : 7;
   const int64_t n = (K * bits / 8 + 1023) / 1024;
   if (bits == 8)
-    return launch_loads<T, 8, kMaxLoadsW8>(n, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-  return launch_loads<T, 4, kMaxLoadsW4>(n, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+    return launch_loads<T, 8, kMaxLoadsW8, kSilu>(n, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+  return launch_loads<T, 4, kMaxLoadsW4, kSilu>(n, x, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
 }
 
 }  // namespace
@@ -439,10 +468,15 @@ bool qmv_dot_covers(int64_t M, int64_t K, int bits) {
 }
 
 int launch_qmv_dot(const void* x, int dtype, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                   const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream) {
-  if (dtype == MFQ_BF16) return launch_type<BF16>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
-  if (dtype == MFQ_F16) return launch_type<F16>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
-  return MFQ_EDTYPE;
+                   const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream,
+                   bool silu) {
+  if (dtype != MFQ_BF16 && dtype != MFQ_F16) return MFQ_EDTYPE;
+  const bool bf = dtype == MFQ_BF16;
+  if (silu)
+    return bf ? launch_type<BF16, true>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream)
+              : launch_type<F16, true>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+  return bf ? launch_type<BF16, false>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream)
+            : launch_type<F16, false>(x, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
 }
 
 }  // namespace mfq

@@ -98,6 +98,11 @@ class QuantizedLinear(torch.nn.Module):
         return core.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
                                      group_size=self.group_size, bits=self.bits, mode=self.mode, bias=self.bias)
 
+    def silu_forward(self, x: torch.Tensor) -> torch.Tensor:
+        """``self(silu(x))``, the activation inside the matvec kernel when ``x`` is one row."""
+        return core.silu_quantized_matmul(x, self.weight, self.scales, self.biases, group_size=self.group_size,
+                                          bits=self.bits, mode=self.mode, bias=self.bias)
+
     @classmethod
     def from_linear(cls, linear_layer: torch.nn.Module, group_size: int | None = None, bits: int | None = None,
                     mode: str = "affine") -> "QuantizedLinear":
@@ -129,6 +134,21 @@ class QuantizedLinear(torch.nn.Module):
         else:
             ql.bias = None
         return ql
+
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """MLX's ``nn.silu``: ``x * sigmoid(x)`` as two operations in ``x``'s dtype."""
+    return core.silu(x)
+
+
+def silu_linear(layer: torch.nn.Module, x: torch.Tensor) -> torch.Tensor:
+    """``layer(nn.silu(x))``, the adaLN modulation call of
+    src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12, as
+    one kernel when ``layer`` is a :class:`QuantizedLinear` and ``x`` one row;
+    the composition otherwise (float linears, LoRA wrappers, more rows)."""
+    if type(layer) is QuantizedLinear:
+        return layer.silu_forward(x)
+    return layer(core.silu(x))
 
 
 def concat_quantized(layers: list[QuantizedLinear]) -> QuantizedLinear:

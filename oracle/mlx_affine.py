@@ -72,6 +72,27 @@ def _from_f32(x: np.ndarray, dtype: int) -> np.ndarray:
     return x.astype(np.float32)
 
 
+def silu_bits(x: np.ndarray, dtype: int = BF16) -> np.ndarray:
+    """MLX's ``nn.silu`` on raw 16-bit storage: ``x * sigmoid(x)`` as two array
+    operations, each rounded to ``dtype`` (python/mlx/nn/layers/activations.py,
+    ``silu``; reached from src/mflux/models/flux/model/flux_transformer/
+    ada_layer_norm_zero.py:12).  The sigmoid is evaluated in float64, with the
+    float32 range of the exponential.
+
+    Parity unpinned against MLX itself (its sigmoid kernel's own rounding is not
+    available here); pinned by tests/test_oracle.py against PyTorch's CPU
+    evaluation of the same two operations, closed-form values and limits."""
+    xf = _to_f32(x, dtype).astype(np.float64)
+    with np.errstate(over="ignore"):
+        e = np.exp(-xf)
+    e = np.where(e > float(np.finfo(np.float32).max), np.inf, e)  # the exponential is a float32 one: x < -88.7 overflows
+    sg = 1.0 / (1.0 + e)
+    sg16 = _to_f32(_from_f32(sg.astype(np.float32), dtype), dtype).astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        prod = (xf * sg16).astype(np.float32)  # exact: two 8- or 11-bit significands
+    return _from_f32(prod, dtype)
+
+
 def _check(group_size: int, bits: int) -> None:
     if group_size not in (32, 64, 128):
         raise ValueError(f"group_size {group_size} not supported")

@@ -20,7 +20,8 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
-                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add"):
+                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add",
+                 "mfq_qmv_silu"):
         assert must in names
 
 
@@ -55,7 +56,7 @@ def test_argument_validation_needs_no_device():
     from mflux_amd import _lib
 
     lib = _lib.load()
-    E = {"dtype": -1, "group": -2, "bits": -3, "shape": -4, "null": -5, "align": -6}
+    E = {"dtype": -1, "group": -2, "bits": -3, "shape": -4, "null": -5, "align": -6, "unsupported": -8}
     buf = ctypes.create_string_buffer(4096 + 64)
     base = (ctypes.addressof(buf) + 15) & ~15
     q = lib.mfq_quantize_affine
@@ -117,6 +118,25 @@ def test_argument_validation_needs_no_device():
     assert add(base, base, _lib.BF16, 4, 8, 24, base, _lib.BF16, None) == E["shape"]
     assert add(base, None, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["null"]
     assert add(base + 8, base, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["align"]
+    # the matvec with the activation inside: one row of 16-bit x, 4 or 8 bits, rows the one-row kernel takes
+    silu = lib.mfq_qmv_silu
+
+    def call_silu(x=base, xd=_lib.BF16, K=3072, wq=base, s=base, b=base, sd=_lib.BF16, N=64, gs=64, bits=8, y=base,
+                  yd=_lib.BF16):
+        return silu(x, xd, K, wq, s, b, sd, None, N, gs, bits, y, yd, None)
+
+    assert call_silu(xd=_lib.F32, sd=_lib.F32) == E["dtype"]
+    assert call_silu(xd=_lib.F16) == E["dtype"]
+    assert call_silu(yd=_lib.F16) == E["dtype"]
+    assert call_silu(K=3000) == E["shape"]
+    assert call_silu(N=0) == E["shape"]
+    assert call_silu(gs=48) == E["group"]
+    assert call_silu(bits=7) == E["bits"]
+    assert call_silu(x=None) == E["null"]
+    assert call_silu(wq=base + 4) == E["align"]
+    assert call_silu(bits=5) == E["unsupported"]
+    assert call_silu(K=8192) == E["unsupported"]            # 8 KiB of 8-bit codes per row
+    assert call_silu(K=8192, bits=4) == E["unsupported"]    # 4 KiB of 4-bit codes per row
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

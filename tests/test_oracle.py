@@ -403,3 +403,61 @@ def test_regression_fixture(oracle):
                       o.BF16, None, 64, bits, y_dtype=o.F32, threads=1)
         ref = data[f"y{bits}"]
         assert (np.abs(y - ref).max(axis=1) <= 1e-5 * np.abs(ref).max(axis=1)).all()
+
+
+# ---------------------------------------------------------------------------
+# silu: the activation in front of the modulation linears
+# ---------------------------------------------------------------------------
+def _all_finite_16(o, dtype):
+    bits = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    f = o._to_f32(bits, dtype)
+    return bits[np.isfinite(f)]
+
+
+@pytest.mark.parametrize("dtype_name", ["bf16", "f16"])
+def test_silu_against_torch_cpu_two_operations(oracle, dtype_name):
+    """Every finite 16-bit value: the oracle (float64 sigmoid, two roundings)
+    against PyTorch's CPU evaluation of the same two operations in the 16-bit
+    type, an independent implementation.  Its float32 exponential may round a
+    sigmoid the other way on a rare value: at most one ulp then, on well under a
+    percent of the values."""
+    import torch
+
+    o = oracle
+    dtype, tdt = (o.BF16, torch.bfloat16) if dtype_name == "bf16" else (o.F16, torch.float16)
+    bits = _all_finite_16(o, dtype)
+    got = o.silu_bits(bits, dtype)
+    x = torch.from_numpy(bits.view(np.int16)).view(tdt)
+    want = (x * torch.sigmoid(x)).view(torch.int16).numpy().view(np.uint16)
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    diff = np.where((got & 0x7FFF) + (want & 0x7FFF) == 0, 0, diff)  # +0 and -0
+    assert diff.max() <= 1
+    assert (diff != 0).mean() < 0.01
+
+
+def test_silu_closed_forms(oracle):
+    o = oracle
+    f = lambda v: float(o.bf16_bits_to_f32(o.silu_bits(o.f32_to_bf16_bits(np.float32([v])), o.BF16))[0])
+    assert f(0.0) == 0.0
+    assert f(1.0) == 0.73046875          # sigmoid(1) = 0.731058..., bfloat16 0.73046875; times 1
+    assert f(64.0) == 64.0 and f(-100.0) == 0.0  # sigmoid saturates: 1, and 0 where the float32 exponential overflows
+    assert f(-64.0) == -64.0 * 1.5859375 * 2.0 ** -93   # sigmoid(-64) = e^-64 = 1.58834 * 2^-93 -> 203/128 * 2^-93
+    # two roundings, not one: somewhere among all values a single rounding of x * sigmoid(x) must differ
+    bits = _all_finite_16(o, o.BF16)
+    x = o.bf16_bits_to_f32(bits).astype(np.float64)
+    with np.errstate(over="ignore"):
+        once = o.f32_to_bf16_bits((x / (1.0 + np.exp(-x))).astype(np.float32))
+    assert (once != o.silu_bits(bits, o.BF16)).any(), "the oracle must round the sigmoid before the product"
+
+
+def test_silu_shape_properties(oracle):
+    o = oracle
+    bits = _all_finite_16(o, o.BF16)
+    x = o.bf16_bits_to_f32(bits)
+    y = o.bf16_bits_to_f32(o.silu_bits(bits, o.BF16))
+    assert np.all(y[x >= 0] >= 0) and np.all(y[x >= 0] <= x[x >= 0])
+    assert np.all(y[x < 0] <= 0) and np.all(y >= np.float32(-0.28))     # minimum of silu is -0.2785
+    big = x > 20
+    assert np.array_equal(y[big], x[big])
+    order = np.argsort(x[x >= 0])
+    assert np.all(np.diff(y[x >= 0][order]) >= 0)                          # monotone on the positive side
