@@ -151,7 +151,7 @@ def silu_linear(layer: torch.nn.Module, x: torch.Tensor) -> torch.Tensor:
     return layer(core.silu(x))
 
 
-def concat_quantized(layers: list[QuantizedLinear]) -> QuantizedLinear:
+def concat_quantized(layers: list[QuantizedLinear], share_storage: bool = False) -> QuantizedLinear:
     """One ``QuantizedLinear`` whose output is the outputs of ``layers`` side by
     side: the packed rows, scales and biases of a weight belong to its output
     feature alone, so stacking them along N needs no requantization.  The q, k
@@ -160,7 +160,16 @@ def concat_quantized(layers: list[QuantizedLinear]) -> QuantizedLinear:
     three calls on the same input) become one launch over three times the
     tiles, which fills the GPU better than three small ones; the caller splits
     the result with ``split`` / slicing (views, no copy).  The inputs are left
-    untouched (their tensors are copied)."""
+    untouched (their tensors are copied) unless ``share_storage`` is set: then
+    every input layer's tensors become views of the stacked ones, so the stack
+    costs no memory and the layers keep working on their own.
+
+    The same serves the adaLN modulation linears of a whole model
+    (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 in
+    every block): all of them take the same ``silu(text_embeddings)``, so
+    ``silu_linear(concat_quantized(all_of_them, share_storage=True), temb)`` at
+    the start of a step is one matvec over gigabytes of weights instead of one
+    launch of 30 to 60 MB per block, each of which pays the launch's fixed cost."""
     if not layers:
         raise ValueError("[concat_quantized] needs at least one layer")
     first = layers[0]
@@ -183,6 +192,16 @@ def concat_quantized(layers: list[QuantizedLinear]) -> QuantizedLinear:
         out.register_buffer("bias", torch.cat(parts, dim=0))
     else:
         out.bias = None
+    if share_storage:
+        row = 0
+        for layer in layers:
+            end = row + layer.output_dims
+            layer._buffers["weight"] = out.weight[row:end]
+            layer._buffers["scales"] = out.scales[row:end]
+            layer._buffers["biases"] = out.biases[row:end]
+            if layer.bias is not None:
+                layer._buffers["bias"] = out.bias[row:end]
+            row = end
     return out
 
 

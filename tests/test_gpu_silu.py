@@ -178,3 +178,25 @@ def test_silu_linear_wrapper(oracle):
     x.requires_grad_(True)   # gradients: the composed, differentiable form
     qnn.silu_linear(q, x).float().sum().backward()
     assert x.grad is not None and bool(torch.isfinite(x.grad).all())
+
+
+def test_modulation_linears_of_several_blocks_as_one_call(oracle):
+    """The modulation linears of all blocks take the same silu(temb): stacked
+    along N (sharing storage with the layers) they give, in one call, bit for
+    bit what each layer gives on its own, since a row's result does not depend
+    on how rows are dealt out."""
+    import mflux_amd
+    from mflux_amd import nn as qnn
+
+    torch.manual_seed(6)
+    layers = [qnn.Linear(3072, n, bias=True, device="cuda", dtype=torch.bfloat16).to_quantized(64, 8)
+              for n in (18432, 18432, 9216, 6144)]
+    for layer in layers:
+        layer.bias.normal_(0, 0.02)
+    temb = (torch.randn(1, 3072, device="cuda") * 2).to(torch.bfloat16)
+    alone = [qnn.silu_linear(layer, temb) for layer in layers]
+    bank = qnn.concat_quantized(layers, share_storage=True)
+    parts = qnn.silu_linear(bank, temb).split([layer.output_dims for layer in layers], dim=-1)
+    for part, ref, layer in zip(parts, alone, layers):
+        assert torch.equal(part, ref)
+        assert torch.equal(qnn.silu_linear(layer, temb), ref)     # the layers still work, now as views of the bank

@@ -197,6 +197,26 @@ def test_concat_quantized_stacks_rows_and_checks_compatibility():
         qnn.concat_quantized([])
 
 
+def test_concat_quantized_share_storage_turns_the_layers_into_views():
+    a = qnn.QuantizedLinear(128, 64, bias=True, bits=8)
+    b = qnn.QuantizedLinear(128, 32, bias=False, bits=8)
+    a.weight.fill_(7), b.weight.fill_(9)
+    a.scales.fill_(0.5), b.scales.fill_(0.25)
+    a.bias.fill_(1.5)
+    fused = qnn.concat_quantized([a, b], share_storage=True)
+    for layer, rows in ((a, slice(0, 64)), (b, slice(64, 96))):
+        for name in ("weight", "scales", "biases"):
+            view, whole = getattr(layer, name), getattr(fused, name)
+            assert view.untyped_storage().data_ptr() == whole.untyped_storage().data_ptr()
+            assert view.is_contiguous() and torch.equal(view.view(torch.uint8), whole[rows].view(torch.uint8))
+    assert a.bias.untyped_storage().data_ptr() == fused.bias.untyped_storage().data_ptr() and b.bias is None
+    assert a.weight.view(torch.int32)[0, 0] == 7 and b.weight.view(torch.int32)[0, 0] == 9
+    assert a.bias.tolist() == [1.5] * 64 and fused.bias.tolist() == [1.5] * 64 + [0.0] * 32
+    assert sorted(a.state_dict()) == ["bias", "biases", "scales", "weight"]     # still the four saved tensors
+    fused.scales[:64].fill_(2.0)                                                # one memory
+    assert a.scales[0, 0] == 2.0
+
+
 def test_quantized_linear_constructor_on_cpu_is_a_placeholder():
     q = qnn.QuantizedLinear(256, 64, bias=True, group_size=None, bits=8)
     assert (q.group_size, q.bits) == (64, 8)
