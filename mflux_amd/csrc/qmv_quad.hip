@@ -116,43 +116,68 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
         reinterpret_cast<const u32x4*>(wbytes + (size_t)q * 4 * row_bytes + lane_woff + 256 * j));
   };
 
-  // The first weight pieces and the first quad's scales are requested before
-  // anything else, so that their latency overlaps the staging of x.
+  // ---- x: the B operands and the slice sums of every lane position are
+  // computed once per workgroup (the four wavefronts share the pieces out) and
+  // kept in LDS.  All of this wavefront's loads of x are requested first and
+  // in one go, the first weight pieces and the first quad's scales right
+  // behind them: loads return in order, so x issued behind the weights, or
+  // piece after piece, would wait for HBM once per piece before the first
+  // quad can start.  Unconditional like every load here: a piece past the
+  // row's end or an activation row past M re-reads a valid one and is dropped.
+  constexpr int kMine = (kLoads + 3) / 4;  // pieces of x a wavefront stages
+  constexpr int kRawWords = BITS == 4 ? 4 : 2;
+  const int x_row = min(li, M - 1);
+  uint32_t raw[kMine][4][kRawWords];
+#pragma unroll
+  for (int i = 0; i < kMine; ++i) {
+    const int j = min(wave + 4 * i, kLoads - 1);
+    const int k0 = (j * 16 + blk) * kCodes;
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) {  // the piece's four words
+      if constexpr (BITS == 4) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(x + (int64_t)x_row * K + k0 + 8 * wd);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) raw[i][wd][e] = v[e];
+      } else {
+        const uint2 v = *reinterpret_cast<const uint2*>(x + (int64_t)x_row * K + k0 + 4 * wd);
+        raw[i][wd][0] = v.x;
+        raw[i][wd][1] = v.y;
+      }
+    }
+  }
   u32x4 ring[kRing];
   const int q_first = has_work ? q_begin : 0;
 #pragma unroll
   for (int j = 0; j < kRing; ++j) ring[j] = load_piece(q_first, j);
   const u32x4 sb_first = load_scales(q_first);
 
-  // ---- x: the B operands and the slice sums of every lane position, computed
-  // once per workgroup (the four wavefronts share the pieces out) and kept in
-  // LDS; every wavefront then reads back the sums of its own lanes
-  for (int j = wave; j < kLoads; j += 4) {
-    const int k0 = (j * 16 + blk) * kCodes;
+#pragma unroll
+  for (int i = 0; i < kMine; ++i) {
+    const int j = wave + 4 * i;
     float sum = 0.f;
 #pragma unroll
-    for (int wd = 0; wd < 4; ++wd) {  // the piece's four words
+    for (int wd = 0; wd < 4; ++wd) {
+      uint32_t v[kRawWords];
+#pragma unroll
+      for (int e = 0; e < kRawWords; ++e) v[e] = li < M ? raw[i][wd][e] : 0u;
       if constexpr (BITS == 4) {
         // word = codes c0..c7; pairs (c0,c4) (c1,c5) | (c2,c6) (c3,c7)
-        u32x4 v = {0, 0, 0, 0};
-        if (li < M) v = *reinterpret_cast<const u32x4*>(x + (int64_t)li * K + k0 + 8 * wd);
-        *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd) * 64 + lane) * 8) =
-            make_uint2((v[0] & 0xffffu) | (v[2] << 16), (v[0] >> 16) | (v[2] & 0xffff0000u));
-        *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd + 1) * 64 + lane) * 8) =
-            make_uint2((v[1] & 0xffffu) | (v[3] << 16), (v[1] >> 16) | (v[3] & 0xffff0000u));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sum += T::to_f32((uint16_t)v[e]) + T::to_f32((uint16_t)(v[e] >> 16));
+        if (j < kLoads) {
+          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd) * 64 + lane) * 8) =
+              make_uint2((v[0] & 0xffffu) | (v[2] << 16), (v[0] >> 16) | (v[2] & 0xffff0000u));
+          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd + 1) * 64 + lane) * 8) =
+              make_uint2((v[1] & 0xffffu) | (v[3] << 16), (v[1] >> 16) | (v[3] & 0xffff0000u));
+        }
       } else {
         // word = codes c0..c3; pairs (c0,c2) (c1,c3)
-        uint2 v = {0, 0};
-        if (li < M) v = *reinterpret_cast<const uint2*>(x + (int64_t)li * K + k0 + 4 * wd);
-        *reinterpret_cast<uint2*>(lds + ((j * kXOps + wd) * 64 + lane) * 8) =
-            make_uint2((v.x & 0xffffu) | (v.y << 16), (v.x >> 16) | (v.y & 0xffff0000u));
-        sum += T::to_f32((uint16_t)v.x) + T::to_f32((uint16_t)(v.x >> 16)) + T::to_f32((uint16_t)v.y) +
-               T::to_f32((uint16_t)(v.y >> 16));
+        if (j < kLoads)
+          *reinterpret_cast<uint2*>(lds + ((j * kXOps + wd) * 64 + lane) * 8) =
+              make_uint2((v[0] & 0xffffu) | (v[1] << 16), (v[0] >> 16) | (v[1] & 0xffff0000u));
       }
+#pragma unroll
+      for (int e = 0; e < kRawWords; ++e) sum += T::to_f32((uint16_t)v[e]) + T::to_f32((uint16_t)(v[e] >> 16));
     }
-    *reinterpret_cast<float*>(lds + kXBytes + (j * 64 + lane) * 4) = sum;
+    if (j < kLoads) *reinterpret_cast<float*>(lds + kXBytes + (j * 64 + lane) * 4) = sum;
   }
   __syncthreads();
   float sx[kLoads];
