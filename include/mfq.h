@@ -122,13 +122,14 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
  *   y       [M, N]                 y_dtype (sb_dtype or MFQ_F32)
  * M <= 16 runs the HBM-bound dequant-GEMV kernel, larger M one of two MFMA
  * GEMM kernels (128-column tiles while 256 x 256 tiles would leave more than
- * half of the compute units idle, 256 x 256 tiles otherwise).  For M > 1 the
+ * half of the compute units idle, 256 x 256 tiles otherwise).  For M > 4 the
  * dequantised weights are rounded once to x_dtype and sums are float32.  For
- * M = 1 (4 and 8 bits) the row of x becomes 15-bit fixed point (one power of
- * two brings its largest magnitude under 2^14: an error of 2^-15 of that
- * magnitude per element, exact for small integers and one-hot rows), the
- * integer dot products with the raw codes are exact, and scale and bias are
- * applied to them in float32; an infinity or NaN in x makes every output NaN.
+ * M <= 4 (4 and 8 bits; shapes the integer kernels take) every row of x
+ * becomes 15-bit fixed point (one power of two per row brings its largest
+ * magnitude under 2^14: an error of 2^-15 of that magnitude per element, exact
+ * for small integers and one-hot rows), the integer products with the raw
+ * codes are exact, and scale and bias are applied to their sums in float32; an
+ * infinity or NaN in a row of x makes every output of that row NaN.
  */
 int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
               const uint32_t* wq, const void* scales, const void* biases,

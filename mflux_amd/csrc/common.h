@@ -138,6 +138,51 @@ struct CodeFloat<F16> {
   }
 };
 
+// ---- a row of 16-bit floats as 15-bit fixed point (the integer matvec kernels) --------------
+// xq = rint(x * 2^e) with 2^e the power of two that brings the row's largest magnitude just
+// under 2^14, split into a signed high and a signed low byte: xq = 256 * xh + xl.
+// Magnitude bits of a 16-bit float: their integer order is the order of the magnitudes.
+__device__ inline int mag_bits(uint32_t pair) { return (int)max(pair & 0x7fffu, (pair >> 16) & 0x7fffu); }
+
+// 2^e as float32 for the exponent field E of the row's largest magnitude
+// (|x| < 2^(E - bias + 1)), so that |x| * 2^e < 2^14; e is kept within what a
+// normal float32 and its reciprocal can hold.
+template <typename T>
+__device__ inline int scale_exponent(int amax_bits);
+template <>
+__device__ inline int scale_exponent<BF16>(int amax_bits) {
+  const int e = 14 - ((amax_bits >> 7) - 127 + 1);
+  return min(max(e, -126), 126);
+}
+template <>
+__device__ inline int scale_exponent<F16>(int amax_bits) {
+  return 14 - ((amax_bits >> 10) - 15 + 1);  // -2 .. 28
+}
+template <typename T>
+__device__ inline bool not_finite(int amax_bits);
+template <>
+__device__ inline bool not_finite<BF16>(int amax_bits) { return (amax_bits >> 7) == 255; }
+template <>
+__device__ inline bool not_finite<F16>(int amax_bits) { return (amax_bits >> 10) == 31; }
+
+__device__ inline float pow2(int e) { return __builtin_bit_cast(float, (uint32_t)(127 + e) << 23); }
+
+// four values of x -> their integer images, high bytes and low bytes packed in k order
+template <typename T>
+__device__ inline void split4(uint32_t p0, uint32_t p1, float mult, uint32_t& hi, uint32_t& lo) {
+  const float f[4] = {lo_f32<T>(p0), hi_f32<T>(p0), lo_f32<T>(p1), hi_f32<T>(p1)};
+  hi = 0;
+  lo = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int q = (int)__builtin_rintf(f[i] * mult);
+    const int l = __builtin_amdgcn_sbfe(q, 0, 8);  // low byte, sign-extended
+    const int h = (q - l) >> 8;
+    lo |= (uint32_t)(l & 0xff) << (8 * i);
+    hi |= (uint32_t)(h & 0xff) << (8 * i);
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Compute units of the current device (256 on an MI355X).

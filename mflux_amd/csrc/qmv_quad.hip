@@ -12,15 +12,25 @@
 // a block are useful: register i of lane (b, j) accumulates row r0+i against
 // activation row j, so up to four activation rows cost what one does, and every
 // load instruction reads 256 contiguous bytes of each of four adjacent rows.
-//   - codes are not converted: one AND-OR per pair of codes makes the exact
-//     16-bit floats "offset + code" (see CodeFloat), the matrix core sums
-//     x * (offset + code) per piece in float32 (a piece lies in one group), and
-//     scale * D + (bias - offset * scale) * sum(x) is the piece's contribution;
-//     scale and bias of row r0+i reach the other lanes of the block as DPP
-//     quad broadcasts;
-//   - the B operands (x, permuted to the order the code pairs come out of a
-//     word) sit in LDS for the whole kernel, one conflict-free 512-byte line per
-//     operand; the scales and biases of the next four rows are fetched with one
+//   - everything runs on integers, on the int8 form of the instruction: every
+//     activation row becomes 15-bit fixed point, xq = rint(x * 2^e) with 2^e
+//     the power of two that brings the row's largest magnitude just under 2^14
+//     (rounding error 2^-15 of that magnitude per element), split into a signed
+//     high and low byte; a word of 8-bit codes goes in as it is, as the signed
+//     bytes code - 128 (one XOR), a word of 4-bit codes as its even and its odd
+//     nibbles (three instructions), each against the high and the low bytes of
+//     x.  Per 16-byte piece (a piece lies in one group) the int32 sums give
+//     D = sum(xq * code) exactly, and scale * D + bias * sum(xq) is the piece's
+//     contribution (the 128 of the 8-bit form joins the bias), scaled back by
+//     2^-e of its activation row at the end.  No code is converted to floating
+//     point and no weight is rounded.  (With 16-bit float operands a bfloat16
+//     8-bit code had to enter as two nibbles: 7 vector and 2 matrix instructions
+//     per word against 1 and 2 now; 3072 -> 18432 at M = 4: 16.6 -> 15.2 us.)
+//     Scale and bias of row r0+i reach the other lanes of the block as DPP quad
+//     broadcasts;
+//   - the B operands (the bytes of xq in the order of the codes of a word,
+//     high bytes and low bytes side by side) sit in LDS for the whole kernel,
+//     one conflict-free 512-byte line per operand pair; the scales and biases of the next four rows are fetched with one
 //     16-byte load per lane and staged through a wavefront-private LDS region;
 //   - weight loads run kRing pieces ahead in a ring of registers, across row
 //     quads; all of them are unconditional (past the end: the wavefront's last
@@ -36,6 +46,8 @@ namespace mfq {
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kDppRowRor4 = 0x124;
 constexpr int kDppRowRor8 = 0x128;
@@ -64,10 +76,8 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
                                                        const uint16_t* __restrict__ bias, void* __restrict__ y,
                                                        int y_is_f32, int M, int N, int K, int gs_shift,
                                                        int quads_per_wave) {
-  using CF = CodeFloat<T>;
   constexpr int kCodes = 128 / BITS;  // codes in one 16-byte piece
-  constexpr int kXOps = kCodes / 4;   // B operands (4 values of x) per piece
-  constexpr float kOffset = BITS == 4 ? CF::kOffset4 : CF::kOffset8;
+  constexpr int kXOps = kCodes / 4;   // B operand pairs (high and low bytes of 4 values of x) per piece
   constexpr int kXBytes = kLoads * kXOps * 512;  // the B operands of one lane set
   static_assert(kLoads % kRing == 0, "ring slots must be known at compile time");
   extern __shared__ __attribute__((aligned(16))) char lds[];  // x operands, slice sums, 4 x 2 scale regions
@@ -100,10 +110,6 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   // where this lane finds the scale of piece (j, blk) of row li inside a region
   const int piece_groups = (16 * kCodes) >> gs_shift;  // groups one load instruction spans
   const int sidx0 = (li * groups + ((blk * kCodes) >> gs_shift)) * 2;
-
-  uint32_t pair_mask = (BITS == 8 && CF::kWholeByte) ? 0x00ff00ffu : 0x000f000fu;
-  uint32_t magic = CF::kNibble, magic_high = CF::kHighMagic;
-  asm volatile("" : "+s"(pair_mask), "+v"(magic), "+v"(magic_high));
 
   auto load_scales = [&](int q) __attribute__((always_inline)) {
     return *reinterpret_cast<const u32x4*>(sb_src + (size_t)q * quad_sb_bytes + sb_off_load);
@@ -151,33 +157,61 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   for (int j = 0; j < kRing; ++j) ring[j] = load_piece(q_first, j);
   const u32x4 sb_first = load_scales(q_first);
 
+  // ---- the integer image of the activation rows: per row one power of two brings its largest
+  // magnitude just under 2^14 (lanes with the same lane % 4 hold the same row)
+  int amax = 0;
+#pragma unroll
+  for (int i = 0; i < kMine; ++i)
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd)
+#pragma unroll
+      for (int e = 0; e < kRawWords; ++e) amax = max(amax, mag_bits(raw[i][wd][e]));
+  amax = max(amax, __builtin_amdgcn_update_dpp(0, amax, kDppRowRor4, 0xf, 0xf, false));
+  amax = max(amax, __builtin_amdgcn_update_dpp(0, amax, kDppRowRor8, 0xf, 0xf, false));
+  amax = max(amax, __builtin_amdgcn_ds_bpermute((lane ^ 16) * 4, amax));
+  amax = max(amax, __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, amax));
+  int* row_amax = reinterpret_cast<int*>(lds + kXBytes + kLoads * 256 + 4 * 2 * kScaleRegion);  // [4 wavefronts][4 rows]
+  if (lane < 4) row_amax[wave * 4 + lane] = amax;
+  __syncthreads();
+  amax = max(max(row_amax[li], row_amax[4 + li]), max(row_amax[8 + li], row_amax[12 + li]));
+  const int e2 = scale_exponent<T>(amax);
+  const float mult = li < M ? pow2(e2) : 0.f;  // activation rows past M: zeros
+  // an infinity or NaN anywhere in a row of x: every output of that row is NaN
+  const float unscale = not_finite<T>(amax) ? __builtin_nanf("") : pow2(-e2);
 #pragma unroll
   for (int i = 0; i < kMine; ++i) {
     const int j = wave + 4 * i;
-    float sum = 0.f;
+    int sum_hi = 0, sum_lo = 0;
 #pragma unroll
     for (int wd = 0; wd < 4; ++wd) {
-      uint32_t v[kRawWords];
-#pragma unroll
-      for (int e = 0; e < kRawWords; ++e) v[e] = li < M ? raw[i][wd][e] : 0u;
       if constexpr (BITS == 4) {
-        // word = codes c0..c7; pairs (c0,c4) (c1,c5) | (c2,c6) (c3,c7)
+        // a weight word holds codes c0..c7; its even nibbles, as bytes, are c0 c2 c4 c6, the odd ones c1 c3 c5 c7.
+        // raw[..][q] = (x[2q], x[2q+1]): even k in the low halves
+        const uint32_t ev0 = (raw[i][wd][0] & 0xffffu) | (raw[i][wd][1] << 16);
+        const uint32_t ev1 = (raw[i][wd][2] & 0xffffu) | (raw[i][wd][3] << 16);
+        const uint32_t od0 = (raw[i][wd][0] >> 16) | (raw[i][wd][1] & 0xffff0000u);
+        const uint32_t od1 = (raw[i][wd][2] >> 16) | (raw[i][wd][3] & 0xffff0000u);
+        uint32_t hi_e, lo_e, hi_o, lo_o;
+        split4<T>(ev0, ev1, mult, hi_e, lo_e);
+        split4<T>(od0, od1, mult, hi_o, lo_o);
         if (j < kLoads) {
-          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd) * 64 + lane) * 8) =
-              make_uint2((v[0] & 0xffffu) | (v[2] << 16), (v[0] >> 16) | (v[2] & 0xffff0000u));
-          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd + 1) * 64 + lane) * 8) =
-              make_uint2((v[1] & 0xffffu) | (v[3] << 16), (v[1] >> 16) | (v[3] & 0xffff0000u));
+          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd) * 64 + lane) * 8) = make_uint2(hi_e, lo_e);
+          *reinterpret_cast<uint2*>(lds + ((j * kXOps + 2 * wd + 1) * 64 + lane) * 8) = make_uint2(hi_o, lo_o);
         }
+        sum_hi = __builtin_amdgcn_sdot4((int)hi_e, 0x01010101, sum_hi, false);
+        sum_hi = __builtin_amdgcn_sdot4((int)hi_o, 0x01010101, sum_hi, false);
+        sum_lo = __builtin_amdgcn_sdot4((int)lo_e, 0x01010101, sum_lo, false);
+        sum_lo = __builtin_amdgcn_sdot4((int)lo_o, 0x01010101, sum_lo, false);
       } else {
-        // word = codes c0..c3; pairs (c0,c2) (c1,c3)
-        if (j < kLoads)
-          *reinterpret_cast<uint2*>(lds + ((j * kXOps + wd) * 64 + lane) * 8) =
-              make_uint2((v[0] & 0xffffu) | (v[1] << 16), (v[0] >> 16) | (v[1] & 0xffff0000u));
+        // a weight word holds codes c0..c3 as its bytes
+        uint32_t hi, lo;
+        split4<T>(raw[i][wd][0], raw[i][wd][1], mult, hi, lo);
+        if (j < kLoads) *reinterpret_cast<uint2*>(lds + ((j * kXOps + wd) * 64 + lane) * 8) = make_uint2(hi, lo);
+        sum_hi = __builtin_amdgcn_sdot4((int)hi, 0x01010101, sum_hi, false);
+        sum_lo = __builtin_amdgcn_sdot4((int)lo, 0x01010101, sum_lo, false);
       }
-#pragma unroll
-      for (int e = 0; e < kRawWords; ++e) sum += T::to_f32((uint16_t)v[e]) + T::to_f32((uint16_t)(v[e] >> 16));
     }
-    if (j < kLoads) *reinterpret_cast<float*>(lds + kXBytes + (j * 64 + lane) * 4) = sum;
+    if (j < kLoads) *reinterpret_cast<float*>(lds + kXBytes + (j * 64 + lane) * 4) = (float)(sum_hi * 256 + sum_lo);
   }
   __syncthreads();
   float sx[kLoads];
@@ -205,35 +239,32 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
       constexpr int slot = j % kRing;
       const float sc = T::to_f32(*reinterpret_cast<const uint16_t*>(sb + j * piece_groups * 2));
       const float bi = T::to_f32(*reinterpret_cast<const uint16_t*>(sb + 512 + j * piece_groups * 2));
-      const float bo = __builtin_fmaf(-kOffset, sc, bi);
+      // 8 bits: code = (code - 128) + 128, and the 128 joins the bias in front of the slice sum
+      const float bo = BITS == 8 ? __builtin_fmaf(128.f, sc, bi) : bi;
+      // exact integer sums of code * xq over the piece, against the high and the low bytes of xq:
       // two accumulation chains, so that a matrix instruction need not wait for the one before it
-      f32x4 d = {0.f, 0.f, 0.f, 0.f}, d2 = {0.f, 0.f, 0.f, 0.f};
+      i32x4 dh = {0, 0, 0, 0}, dl = {0, 0, 0, 0};
 #pragma unroll
       for (int wd = 0; wd < 4; ++wd) {
         const uint32_t w = ring[slot][wd];
         if constexpr (BITS == 4) {
-          const uint2 a0 = make_uint2((w & pair_mask) | magic, ((w >> 4) & pair_mask) | magic);
-          const uint2 a1 = make_uint2(((w >> 8) & pair_mask) | magic, ((w >> 12) & pair_mask) | magic);
-          d = CF::mfma4(a0, *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd) * 512), d);
-          d2 = CF::mfma4(a1, *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd + 1) * 512), d2);
-        } else if constexpr (CF::kWholeByte) {
-          const uint2 a = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
-          const uint2 xb = *reinterpret_cast<const uint2*>(xops + (j * kXOps + wd) * 512);
-          if (wd & 1) {
-            d2 = CF::mfma4(a, xb, d2);
-          } else {
-            d = CF::mfma4(a, xb, d);
-          }
+          const int ev = (int)(w & 0x0f0f0f0fu), od = (int)((w >> 4) & 0x0f0f0f0fu);
+          const uint2 xe = *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd) * 512);
+          const uint2 xo = *reinterpret_cast<const uint2*>(xops + (j * kXOps + 2 * wd + 1) * 512);
+          dh = __builtin_amdgcn_mfma_i32_4x4x4i8(ev, (int)xe.x, dh, 0, 0, 0);
+          dl = __builtin_amdgcn_mfma_i32_4x4x4i8(ev, (int)xe.y, dl, 0, 0, 0);
+          dh = __builtin_amdgcn_mfma_i32_4x4x4i8(od, (int)xo.x, dh, 0, 0, 0);
+          dl = __builtin_amdgcn_mfma_i32_4x4x4i8(od, (int)xo.y, dl, 0, 0, 0);
         } else {
-          const uint2 lo = make_uint2((w & pair_mask) | magic, ((w >> 8) & pair_mask) | magic);
-          const uint2 hi = make_uint2(((w >> 4) & pair_mask) | magic_high, ((w >> 12) & pair_mask) | magic_high);
+          const int c = (int)(w ^ 0x80808080u);  // code - 128 as signed bytes
           const uint2 xb = *reinterpret_cast<const uint2*>(xops + (j * kXOps + wd) * 512);
-          d = CF::mfma4(lo, xb, d);
-          d2 = CF::mfma4(hi, xb, d2);
+          dh = __builtin_amdgcn_mfma_i32_4x4x4i8(c, (int)xb.x, dh, 0, 0, 0);
+          dl = __builtin_amdgcn_mfma_i32_4x4x4i8(c, (int)xb.y, dl, 0, 0, 0);
         }
       }
+      float d[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) d[e] += d2[e];
+      for (int e = 0; e < 4; ++e) d[e] = (float)(dh[e] * 256 + dl[e]);
       // refill the slot: the piece kRing further on, in this quad or the next
       if constexpr (j + kRing < kLoads) {
         ring[slot] = load_piece(q, j + kRing);
@@ -265,7 +296,7 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
       v += dpp_f32<kDppRowRor8>(v);
       v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) * 4, __builtin_bit_cast(int, v)));
       v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, __builtin_bit_cast(int, v)));
-      tot[i] = v;
+      tot[i] = v * unscale;
     }
     if (lane < M) {  // lane m holds y[m, r0..r0+3]
       const int64_t r0 = (int64_t)q * 4;
@@ -297,7 +328,7 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
   auto kernel = qmv_quad_kernel<T, BITS, kLoads, kRing>;
   constexpr int kXOps = 128 / BITS / 4;
-  constexpr int kLds = kLoads * kXOps * 512 + kLoads * 256 + 4 * 2 * kScaleRegion;
+  constexpr int kLds = kLoads * kXOps * 512 + kLoads * 256 + 4 * 2 * kScaleRegion + 64;  // + the rows' largest magnitudes
   static int blocks_per_cu = 0;
   if (blocks_per_cu == 0) {
     if (kLds > 48 * 1024 &&
