@@ -167,20 +167,20 @@ __device__ inline bool not_finite<F16>(int amax_bits) { return (amax_bits >> 10)
 
 __device__ inline float pow2(int e) { return __builtin_bit_cast(float, (uint32_t)(127 + e) << 23); }
 
-// four values of x -> their integer images, high bytes and low bytes packed in k order
+// four values of x -> their integer images, high bytes and low bytes packed in k order.
+// xq = 256 * h + l with l the low byte read as signed, so h is the high byte of xq + 128;
+// |xq| <= 2^14 fits the 16-bit halves the bytes are picked from.
 template <typename T>
 __device__ inline void split4(uint32_t p0, uint32_t p1, float mult, uint32_t& hi, uint32_t& lo) {
-  const float f[4] = {lo_f32<T>(p0), hi_f32<T>(p0), lo_f32<T>(p1), hi_f32<T>(p1)};
-  hi = 0;
-  lo = 0;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int q = (int)__builtin_rintf(f[i] * mult);
-    const int l = __builtin_amdgcn_sbfe(q, 0, 8);  // low byte, sign-extended
-    const int h = (q - l) >> 8;
-    lo |= (uint32_t)(l & 0xff) << (8 * i);
-    hi |= (uint32_t)(h & 0xff) << (8 * i);
-  }
+  typedef short s16x2 __attribute__((ext_vector_type(2)));
+  const int q0 = (int)__builtin_rintf(lo_f32<T>(p0) * mult), q1 = (int)__builtin_rintf(hi_f32<T>(p0) * mult);
+  const int q2 = (int)__builtin_rintf(lo_f32<T>(p1) * mult), q3 = (int)__builtin_rintf(hi_f32<T>(p1) * mult);
+  const s16x2 q01 = __builtin_amdgcn_cvt_pk_i16(q0, q1), q23 = __builtin_amdgcn_cvt_pk_i16(q2, q3);
+  const s16x2 half = {128, 128};
+  const s16x2 t01 = q01 + half, t23 = q23 + half;
+  // byte selectors: 0..3 name the bytes of the second operand, 4..7 those of the first
+  lo = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, q23), __builtin_bit_cast(uint32_t, q01), 0x06040200u);
+  hi = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, t23), __builtin_bit_cast(uint32_t, t01), 0x07050301u);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
