@@ -94,12 +94,11 @@ struct DotRow {
   u32x4 w[kLoads];
   uint16_t s[kLoads], b[kLoads];  // per-lane loads (when `kCoop` is off)
   uint32_t sb;                    // cooperative load: lanes 0..31 hold scale pairs, 32..63 bias pairs
-  uint16_t bias;
 
   // Every load is unconditional (addresses past the row's end are clamped into
   // it; what they bring meets zeros of x), so that the number of loads in
   // flight is known when the kernel waits for older ones.
-  __device__ inline void issue(const char* wq, const uint16_t* scales, const uint16_t* biases, const uint16_t* bias_v,
+  __device__ inline void issue(const char* wq, const uint16_t* scales, const uint16_t* biases,
                                int64_t row, int row_bytes, int groups, const int (&piece)[kLoads],
                                const int (&grp)[kLoads], int lane) {
     const char* wrow = wq + row * row_bytes;
@@ -118,7 +117,6 @@ struct DotRow {
 #pragma unroll
     for (int j = 0; j < kLoads; ++j)
       w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wrow + piece[j]));
-    bias = (bias_v ? bias_v + row : srow)[0];  // without a bias: any readable address, the value is not used
   }
 };
 
@@ -175,9 +173,12 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
   const int64_t row_begin = (int64_t)wave_id * rows_per_wave + min(wave_id, extra_rows);
   const int64_t row_end = row_begin + rows_per_wave + (wave_id < extra_rows ? 1 : 0);
   const char* wbytes = reinterpret_cast<const char*>(wq);
+  // the layer's bias of the row whose result this lane will keep (lane i: the i-th row of the run), requested
+  // ahead of the rows so that it has arrived with the first of them (loads return in order)
+  const uint16_t lane_bias = (bias ? bias : scales)[min(row_begin + lane, (int64_t)N - 1)];
   R regs[2];
   // (a wavefront without rows, which a grid rounded up to whole workgroups can leave, re-reads the last row)
-  regs[0].issue(wbytes, scales, biases, bias, min(row_begin, (int64_t)N - 1), row_bytes, groups, piece, grp, lane);
+  regs[0].issue(wbytes, scales, biases, min(row_begin, (int64_t)N - 1), row_bytes, groups, piece, grp, lane);
 
   if constexpr (kSilu) {  // the activation in front of the linear, on the values as they arrive
 #pragma unroll
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
 
   if (row_begin >= row_end) return;  // behind the last barrier
 
-  uint32_t kept = 0;  // lane i: the finished output of the i-th row of the run in hand
+  float kept = 0.f;  // lane i: the sum of the i-th row of the run in hand
   auto consume = [&](const R& regs, int64_t row) __attribute__((always_inline)) {
     float tot = 0.f;
 #pragma unroll
@@ -295,24 +296,24 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
     }
     // every lane holds the row's result; lane (row - row_begin) % 64 keeps it until flush()
     // (selects, not branches: the loop body stays one block, which keeps the requests where they are put)
-    const float v = wave_sum(tot) * unscale;
-    const float bv = T::to_f32(regs.bias);
-    const float v32 = bias ? v + bv : v;
-    const uint16_t h0 = T::from_f32(v);
-    const uint16_t h1 = T::from_f32(T::to_f32(h0) + bv);  // second rounding, as a separate add on the 16-bit result
-    const uint32_t out = y_is_f32 ? __builtin_bit_cast(uint32_t, v32) : (uint32_t)(bias ? h1 : h0);
-    kept = lane == (int)((row - row_begin) & 63) ? out : kept;
+    // (scaling back, the layer's bias and the roundings wait for flush(), where every lane does its own row's)
+    const float v = wave_sum(tot);
+    kept = lane == (int)((row - row_begin) & 63) ? v : kept;
   };
   // Stores the results of rows [first, first + count), count <= 64, one per lane.
   // Results leave the wavefront once, at its end, and not row by row: a store
   // in flight between the loads would make every wait for a load a wait for
   // everything (loads and stores share one counter and may overtake each other).
   auto flush = [&](int64_t first, int count) {
+    const float v = kept * unscale;
+    const float bv = T::to_f32(lane_bias);
     if (lane < count) {
       if (y_is_f32) {
-        reinterpret_cast<uint32_t*>(y)[first + lane] = kept;
+        reinterpret_cast<float*>(y)[first + lane] = bias ? v + bv : v;
       } else {
-        reinterpret_cast<uint16_t*>(y)[first + lane] = (uint16_t)kept;
+        const uint16_t h0 = T::from_f32(v);
+        const uint16_t h1 = T::from_f32(T::to_f32(h0) + bv);  // second rounding, as a separate add on the 16-bit result
+        reinterpret_cast<uint16_t*>(y)[first + lane] = bias ? h1 : h0;
       }
     }
   };
@@ -330,17 +331,17 @@ __global__ __launch_bounds__(256) void qmv_dot_kernel(const uint16_t* __restrict
     for (int64_t row = first; row < row_end; row += 2) {
       // the requests stay between the arithmetic of two rows, in front of the waits for the older row
       __builtin_amdgcn_sched_barrier(0);
-      regs[kP ^ 1].issue(wbytes, scales, biases, bias, row + 1, row_bytes, groups, piece, grp, lane);
+      regs[kP ^ 1].issue(wbytes, scales, biases, row + 1, row_bytes, groups, piece, grp, lane);
       __builtin_amdgcn_sched_barrier(0);
       consume(regs[kP], row);
       __builtin_amdgcn_sched_barrier(0);
-      regs[kP].issue(wbytes, scales, biases, bias, min(row + 2, last), row_bytes, groups, piece, grp, lane);
+      regs[kP].issue(wbytes, scales, biases, min(row + 2, last), row_bytes, groups, piece, grp, lane);
       __builtin_amdgcn_sched_barrier(0);
       consume(regs[kP ^ 1], row + 1);
     }
   };
   if ((row_end - row_begin) & 1) {
-    regs[1].issue(wbytes, scales, biases, bias, min(row_begin + 1, last), row_bytes, groups, piece, grp, lane);
+    regs[1].issue(wbytes, scales, biases, min(row_begin + 1, last), row_bytes, groups, piece, grp, lane);
     __builtin_amdgcn_sched_barrier(0);
     consume(regs[0], row_begin);
     pairs(std::integral_constant<int, 1>{}, row_begin + 1);
