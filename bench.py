@@ -312,20 +312,22 @@ def main():
             state["i"] += 1
             mflux_amd.quantized_matmul(mflux_amd.silu(temb16), wqg, sg, bg, group_size=GS, bits=bits_g, bias=bias)
 
-        if bits_g == 8:
-            # every double block's two modulation linears of a FLUX.1 step as one call: they all take the
-            # same silu(temb), so their packed weights stack along N (38 x 18432 rows, 2.3 GB: cold by size)
-            picks = [bufs[i % n_buf] for i in range(38)]
-            wq_all, s_all, b_all = (torch.cat([p[j] for p in picks]) for j in range(3))
-            bias_all = bias.repeat(38)
-            call_all = lambda: mflux_amd.silu_quantized_matmul(temb16, wq_all, s_all, b_all, group_size=GS,
-                                                               bits=bits_g, bias=bias_all)
-            call_all()
-            ms = event_ms(call_all, 10, torch)
-            nbytes = qmm_bytes(1, Kg, 38 * Ng, bits_g, bias=True)
-            res["M1_38_linears_one_call"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
-                                             "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": nbytes}
-            del picks, wq_all, s_all, b_all, bias_all
+        # all modulation linears of a step as one call: they all take the same silu(temb), so their packed
+        # weights stack along N.  W8: the 38 linears of FLUX.1's double blocks (2.3 GB); W4: the 120 of
+        # Qwen-Image's 60 blocks (3.8 GB).  Cold by size.
+        n_stack = 38 if bits_g == 8 else 120
+        picks = [bufs[i % n_buf] for i in range(n_stack)]
+        wq_all, s_all, b_all = (torch.cat([p[j] for p in picks]) for j in range(3))
+        bias_all = bias.repeat(n_stack)
+        call_all = lambda: mflux_amd.silu_quantized_matmul(temb16, wq_all, s_all, b_all, group_size=GS,
+                                                           bits=bits_g, bias=bias_all)
+        call_all()
+        ms = event_ms(call_all, 10, torch)
+        nbytes = qmm_bytes(1, Kg, n_stack * Ng, bits_g, bias=True)
+        res[f"M1_{n_stack}_linears_one_call"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                                                 "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                                 "bytes": nbytes}
+        del picks, wq_all, s_all, b_all, bias_all
         res["M1_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
                                "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
         gemv[f"w{bits_g}"] = res
