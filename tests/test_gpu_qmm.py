@@ -230,6 +230,57 @@ def test_qmv_one_row_fixed_point_image_of_x(oracle, bits):
     assert np.all(np.isnan(run(xinf)))
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M", [2, 3, 4])
+def test_qmv_four_rows_fixed_point_images_of_x(oracle, bits, M):
+    """The four-rows kernel gives every activation row its own power-of-two
+    scale.  Small integers stay exact whatever the other rows hold; rows of very
+    different magnitude do not disturb each other; a zero row gives the bias;
+    an infinity makes its own row NaN and leaves the others as they were."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    rng = np.random.default_rng(77 + 10 * bits + M)
+    K, N = 3072, 256
+    n_bins = 2 ** bits - 1
+    codes = rng.integers(0, n_bins + 1, (N, K)).astype(np.float32)
+    codes[:, ::64] = 0
+    codes[:, 1::64] = n_bins          # every group spans 0..n_bins: the dequantised weight is the code
+    wq, s, b = o.c_quantize(o.f32_to_bf16_bits(codes), o.BF16, 64, bits)
+    assert np.array_equal(o.dequantize_exact(wq, s, b, o.BF16, 64, bits), codes)
+    dev = lambda a: to_dev(a, o.BF16)
+    run = lambda xb, **kw: mflux_amd.quantized_matmul(dev(xb).float(), u32_to_dev(wq), dev(s), dev(b), group_size=64,
+                                                      bits=bits, **kw).cpu().numpy().astype(np.float64)
+    c64 = codes.astype(np.float64)
+    # small integers in every row, each row at its own magnitude (powers of two keep them exact in bfloat16)
+    xi = rng.integers(-3, 4, (M, K)).astype(np.float32) * (2.0 ** np.arange(0, 6 * M, 6, dtype=np.float32))[:, None]
+    assert np.array_equal(run(o.f32_to_bf16_bits(xi)), xi.astype(np.float64) @ c64.T)
+    # rows 1e-12 ... 1e20 side by side: each within its own bound
+    mags = np.array([1e-12, 1.0, 1e20, 1e-3][:M], dtype=np.float64)[:, None]
+    xb = o.f32_to_bf16_bits((rng.standard_normal((M, K)) * mags).astype(np.float32))
+    xf = o.bf16_bits_to_f32(xb).astype(np.float64)
+    ref = xf @ c64.T
+    got = run(xb)
+    bound = 2.0 ** -15 * np.abs(xf).max(axis=1, keepdims=True) * np.abs(c64).sum(axis=1)[None, :] + 2.0 ** -20 * np.abs(ref)
+    assert np.all(np.isfinite(got)) and np.all(np.abs(got - ref) <= bound)
+    # a zero row gives the bias exactly, next to rows that are not zero
+    bias = o.f32_to_bf16_bits(seeded(78, 2, (N,), 1.0))
+    xz = xb.copy()
+    xz[0] = 0
+    got = run(xz, bias=dev(bias))
+    assert np.array_equal(got[0], o.bf16_bits_to_f32(bias).astype(np.float64))
+    # an infinity: its row is NaN, the other rows unchanged
+    base = run(xb)
+    xinf = xb.copy()
+    xinf[1, 1000] = 0x7f80
+    got = run(xinf)
+    assert np.all(np.isnan(got[1]))
+    keep = [m for m in range(M) if m != 1]
+    assert np.array_equal(got[keep], base[keep])
+
+
+
 @pytest.mark.parametrize("N", [1, 2, 3, 5, 63, 262144 + 8])
 def test_qmv_one_row_run_lengths(oracle, N):
     """Rows are dealt to wavefronts in runs of up to 64 (a lane keeps one
