@@ -330,6 +330,9 @@ def main():
         del picks, wq_all, s_all, b_all, bias_all
         res["M1_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
                                "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
+        temb16 = torch.randn(4, Kg, device=dev, generator=gen).to(torch.bfloat16)  # the same for a batch of four
+        res["M4_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
+                               "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
         gemv[f"w{bits_g}"] = res
         del bufs
 

@@ -160,24 +160,26 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  size_t workspace_bytes, void* stream);
 
 /*
- * y[n] = sum_k silu(x)[k] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs]) (+ bias[n]):
+ * y[m, n] = sum_k silu(x)[m, k] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs]) (+ bias[n]):
  * the adaLN modulation call linear(nn.silu(text_embeddings)) of every
- * transformer block as one kernel, for one row of x
+ * transformer block as one kernel, for one to four rows of x (the batch)
  *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12
  *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero_single.py:12
  *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_continuous.py:15
  * (the reference runs nn.silu as an elementwise kernel of its own in front
  * of the quantized matmul).  silu(x) = x * sigmoid(x) with the sigmoid and
  * the product each rounded to x_dtype, as the two operations of MLX's nn.silu
- * on a 16-bit array round; the rounded row then goes through exactly what
- * mfq_qmm_t does for M = 1.  Arguments as for mfq_qmm_t with M = 1.
+ * on a 16-bit array round; the rounded rows then go through exactly what
+ * mfq_qmm_t does for M <= 4.  Arguments as for mfq_qmm_t.
  * MFQ_EUNSUPPORTED when no fused kernel takes the shape (bits other than 4
- * and 8, rows of more than 6 KiB of 8-bit or 3 KiB of 4-bit codes): apply the
- * activation separately and call mfq_qmm_t.
+ * and 8; M = 1 with rows of more than 6 KiB of 8-bit or 3 KiB of 4-bit codes;
+ * M = 2..4 outside what the four-rows kernel takes: K > 4096, N not a multiple
+ * of 4, rows that are not 1, 2, 3, 4, 6, 8, 12 or 16 times 256 bytes; M > 4):
+ * apply the activation separately and call mfq_qmm_t.
  */
-int mfq_qmv_silu(const void* x, int x_dtype, int64_t K, const uint32_t* wq, const void* scales,
-                 const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size,
-                 int bits, void* y, int y_dtype, void* stream);
+int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
+                 const void* scales, const void* biases, int sb_dtype, const void* bias, int64_t N,
+                 int group_size, int bits, void* y, int y_dtype, void* stream);
 
 /*
  * A quantized linear layer with LoRA adapters on it in one call:

@@ -28,7 +28,7 @@ SIGNATURES = {
                             ctypes.c_size_t, _PTR]),
     "mfq_qmm_t_low_rank": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _PTR,
                                   _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),
-    "mfq_qmv_silu": (_INT, [_PTR, _INT, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmv_silu": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_low_rank_add": (_INT, [_PTR, _PTR, _INT, _I64, _I64, _I64, _PTR, _INT, _PTR]),
 }
 

@@ -258,9 +258,9 @@ def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor
     src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 (and
     ada_layer_norm_zero_single.py:12, ada_layer_norm_continuous.py:15).
 
-    For one row of 16-bit ``x`` against 4- or 8-bit weights the activation runs
-    inside the matvec kernel, where the row is converted anyway
-    (``mfq_qmv_silu``); for any other call it is :func:`silu`, an elementwise
+    For one to four rows of 16-bit ``x`` against 4- or 8-bit weights the
+    activation runs inside the matvec kernel, where the rows are converted
+    anyway (``mfq_qmv_silu``); for any other call it is :func:`silu`, an elementwise
     pass, in front of :func:`quantized_matmul`.  Both round the sigmoid and the
     product to ``x``'s dtype.  Not differentiable in its fused form: with
     gradients enabled on ``x`` or ``bias`` the composed form runs.
@@ -269,8 +269,8 @@ def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor
     _check_group_bits("quantized_matmul", group_size, bits)
     needs_grad = torch.is_grad_enabled() and (x.requires_grad or (bias is not None and bias.requires_grad))
     K = w.shape[-1] * 32 // bits
-    one_row = x.ndim >= 1 and x.shape[-1] == K and x.numel() == K
-    fusable = (one_row and not needs_grad and w.ndim == 2 and bits in MATMUL_KERNEL_BITS
+    M = x.numel() // K if x.ndim >= 1 and x.shape[-1] == K else 0
+    fusable = (1 <= M <= 4 and not needs_grad and w.ndim == 2 and bits in MATMUL_KERNEL_BITS
                and x.dtype == scales.dtype and x.dtype in (torch.bfloat16, torch.float16))
     if fusable:
         _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
@@ -281,12 +281,12 @@ def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor
             if bias.shape != (N,):
                 raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
             bias = bias.to(x.dtype).contiguous()
-        x1 = x.reshape(K).contiguous()
+        x1 = x.reshape(M, K).contiguous()
         w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
-        y = torch.empty((1, N), dtype=x.dtype, device=x.device)
+        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
         with torch.cuda.device(x.device):
             rc = _lib.load().mfq_qmv_silu(
-                x1.data_ptr(), _DTYPE_CODE[x.dtype], K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
+                x1.data_ptr(), _DTYPE_CODE[x.dtype], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
                 _DTYPE_CODE[x.dtype], bias.data_ptr() if bias is not None else None, N, group_size, bits,
                 y.data_ptr(), _DTYPE_CODE[x.dtype], _stream_ptr(x.device))
         if rc != _lib.MFQ_EUNSUPPORTED:

@@ -140,19 +140,24 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
                          workspace_bytes, (hipStream_t)stream, low_rank);
 }
 
-int mfq_qmv_silu(const void* x, int x_dtype, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                 int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y, int y_dtype,
-                 void* stream) {
+int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                 const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
+                 int y_dtype, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
   if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
-  if (N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
-  if (N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
   if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
   if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
-  if ((bits != 4 && bits != 8) || !mfq::qmv_dot_covers(1, K, bits)) return MFQ_EUNSUPPORTED;
-  return mfq::launch_qmv_dot(x, x_dtype, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
-                             (hipStream_t)stream, true);
+  if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;
+  if (mfq::qmv_dot_covers(M, K, bits))
+    return mfq::launch_qmv_dot(x, x_dtype, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                               (hipStream_t)stream, true);
+  if (M >= 2 && M <= 4 && mfq::qmv_quad_covers(M, K, N, group_size, bits, scales, biases, bias, y, y_dtype))
+    return mfq::launch_qmv_quad(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                (hipStream_t)stream, true);
+  return MFQ_EUNSUPPORTED;
 }
 
 int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank, void* y, int y_dtype,

@@ -183,6 +183,25 @@ __device__ inline void split4(uint32_t p0, uint32_t p1, float mult, uint32_t& hi
   hi = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, t23), __builtin_bit_cast(uint32_t, t01), 0x07050301u);
 }
 
+// SiLU of a pair of 16-bit floats as MLX's nn.silu computes it on that type,
+// x * sigmoid(x) with the sigmoid rounded to the type before the product
+// (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 feeds
+// nn.silu(text_embeddings) to the modulation linear).
+template <typename T>
+__device__ inline uint32_t silu_pair(uint32_t pair) {
+  uint32_t out = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const float v = h ? hi_f32<T>(pair) : lo_f32<T>(pair);
+    // hardware exponential and reciprocal (one ulp each, far inside the rounding to 16 bits that follows);
+    // a denormal exponential flushed to 0 leaves the sigmoid at 1, an overflowing one makes it 0
+    const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
+    const float sg = T::to_f32(T::from_f32(__builtin_amdgcn_rcpf(1.f + e)));
+    out |= (uint32_t)T::from_f32(v * sg) << (16 * h);
+  }
+  return out;
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Compute units of the current device (256 on an MI355X).
@@ -231,9 +250,10 @@ int launch_qmv_odd(const void* x, int dtype, int64_t M, int64_t K, const uint32_
 // four weight rows at a time, M <= 4 (qmv_quad_covers() says whether it takes a shape)
 bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* scales, const void* biases,
                      const void* bias, const void* y, int y_dtype);
+// `silu`: the rows that meet the weights are silu(x), each value rounded to `dtype`
 int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                    hipStream_t stream);
+                    hipStream_t stream, bool silu = false);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
 // low_rank: accumulated with the product by both GEMM kernels (a second kernel

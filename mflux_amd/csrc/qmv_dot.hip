@@ -70,25 +70,6 @@ __device__ inline int wave_max(int v) {
              max(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
-// SiLU of a pair of 16-bit floats as MLX's nn.silu computes it on that type,
-// x * sigmoid(x) with the sigmoid rounded to the type before the product
-// (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 feeds
-// nn.silu(text_embeddings) to the modulation linear).
-template <typename T>
-__device__ inline uint32_t silu_pair(uint32_t pair) {
-  uint32_t out = 0;
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const float v = h ? hi_f32<T>(pair) : lo_f32<T>(pair);
-    // hardware exponential and reciprocal (one ulp each, far inside the rounding to 16 bits that follows);
-    // a denormal exponential flushed to 0 leaves the sigmoid at 1, an overflowing one makes it 0
-    const float e = __builtin_amdgcn_exp2f(v * -1.44269504088896341f);
-    const float sg = T::to_f32(T::from_f32(__builtin_amdgcn_rcpf(1.f + e)));
-    out |= (uint32_t)T::from_f32(v * sg) << (16 * h);
-  }
-  return out;
-}
-
 template <typename T, int BITS, int kLoads, bool kCoop>
 struct DotRow {
   u32x4 w[kLoads];

@@ -69,7 +69,7 @@ __device__ inline void for_each_index(F&& f) {
 constexpr int kScaleRegion = 1024;  // per wavefront and buffer: 512 bytes of scales, 512 of biases
 
 // kLoads: 256-byte pieces per weight row (K * BITS / 8 / 256); kRing divides it.
-template <typename T, int BITS, int kLoads, int kRing>
+template <typename T, int BITS, int kLoads, int kRing, bool kSilu>
 __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq,
                                                        const uint16_t* __restrict__ scales,
                                                        const uint16_t* __restrict__ biases,
@@ -156,6 +156,15 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
 #pragma unroll
   for (int j = 0; j < kRing; ++j) ring[j] = load_piece(q_first, j);
   const u32x4 sb_first = load_scales(q_first);
+
+  if constexpr (kSilu) {  // the activation in front of the linear, on the values as they arrive
+#pragma unroll
+    for (int i = 0; i < kMine; ++i)
+#pragma unroll
+      for (int wd = 0; wd < 4; ++wd)
+#pragma unroll
+        for (int e = 0; e < kRawWords; ++e) raw[i][wd][e] = silu_pair<T>(raw[i][wd][e]);
+  }
 
   // ---- the integer image of the activation rows: per row one power of two brings its largest
   // magnitude just under 2^14 (lanes with the same lane % 4 hold the same row)
@@ -323,10 +332,10 @@ __global__ __launch_bounds__(256, 4) void qmv_quad_kernel(const uint16_t* __rest
   }
 }
 
-template <typename T, int BITS, int kLoads, int kRing>
+template <typename T, int BITS, int kLoads, int kRing, bool kSilu>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
-  auto kernel = qmv_quad_kernel<T, BITS, kLoads, kRing>;
+  auto kernel = qmv_quad_kernel<T, BITS, kLoads, kRing, kSilu>;
   constexpr int kXOps = 128 / BITS / 4;
   constexpr int kLds = kLoads * kXOps * 512 + kLoads * 256 + 4 * 2 * kScaleRegion + 64;  // + the rows' largest magnitudes
   static int blocks_per_cu = 0;
@@ -355,13 +364,13 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
-template <typename T, int BITS>
+template <typename T, int BITS, bool kSilu>
 int launch_loads(int64_t loads, const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                  const void* biases, const void* bias, int64_t N, int gs_shift, void* y, int y_dtype,
                  hipStream_t stream) {
 #define MFQ_QUAD_CASE(L, R)                                                                                      \
   case L:                                                                                                        \
-    return launch_kernel<T, BITS, L, R>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream)
+    return launch_kernel<T, BITS, L, R, kSilu>(x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream)
   switch (loads) {
     MFQ_QUAD_CASE(1, 1);
     MFQ_QUAD_CASE(2, 2);
@@ -397,22 +406,28 @@ bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const vo
          aligned16(scales) && aligned16(biases) && (reinterpret_cast<uintptr_t>(y) & y_mask) == 0;
 }
 
-int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
-                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                    hipStream_t stream) {
+namespace {
+template <typename T, bool kSilu>
+int launch_type(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, hipStream_t stream) {
   const int gs_shift = gs == 32 ? 5 : gs == 64 ? 6 : 7;
   const int64_t loads = K * bits / 8 / 256;
-  if (dtype == MFQ_BF16) {
-    if (bits == 4)
-      return launch_loads<BF16, 4>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-    return launch_loads<BF16, 8>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-  }
-  if (dtype == MFQ_F16) {
-    if (bits == 4)
-      return launch_loads<F16, 4>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-    return launch_loads<F16, 8>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
-  }
-  return MFQ_EDTYPE;
+  if (bits == 4)
+    return launch_loads<T, 4, kSilu>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+  return launch_loads<T, 8, kSilu>(loads, x, M, K, wq, scales, biases, bias, N, gs_shift, y, y_dtype, stream);
+}
+}  // namespace
+
+int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                    hipStream_t stream, bool silu) {
+  if (dtype != MFQ_BF16 && dtype != MFQ_F16) return MFQ_EDTYPE;
+  const bool bf = dtype == MFQ_BF16;
+  if (silu)
+    return bf ? launch_type<BF16, true>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream)
+              : launch_type<F16, true>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+  return bf ? launch_type<BF16, false>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream)
+            : launch_type<F16, false>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
 }
 
 }  // namespace mfq

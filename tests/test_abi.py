@@ -121,9 +121,9 @@ def test_argument_validation_needs_no_device():
     # the matvec with the activation inside: one row of 16-bit x, 4 or 8 bits, rows the one-row kernel takes
     silu = lib.mfq_qmv_silu
 
-    def call_silu(x=base, xd=_lib.BF16, K=3072, wq=base, s=base, b=base, sd=_lib.BF16, N=64, gs=64, bits=8, y=base,
-                  yd=_lib.BF16):
-        return silu(x, xd, K, wq, s, b, sd, None, N, gs, bits, y, yd, None)
+    def call_silu(x=base, xd=_lib.BF16, M=1, K=3072, wq=base, s=base, b=base, sd=_lib.BF16, N=64, gs=64, bits=8,
+                  y=base, yd=_lib.BF16):
+        return silu(x, xd, M, K, wq, s, b, sd, None, N, gs, bits, y, yd, None)
 
     assert call_silu(xd=_lib.F32, sd=_lib.F32) == E["dtype"]
     assert call_silu(xd=_lib.F16) == E["dtype"]
@@ -137,6 +137,10 @@ def test_argument_validation_needs_no_device():
     assert call_silu(bits=5) == E["unsupported"]
     assert call_silu(K=8192) == E["unsupported"]            # 8 KiB of 8-bit codes per row
     assert call_silu(K=8192, bits=4) == E["unsupported"]    # 4 KiB of 4-bit codes per row
+    assert call_silu(M=0) == E["shape"]
+    assert call_silu(M=5) == E["unsupported"]               # more rows than the fused kernels take
+    assert call_silu(M=3, N=66) == E["unsupported"]         # the four-rows kernel wants whole quads of weight rows
+    assert call_silu(M=2, K=8192, bits=4) == E["unsupported"]
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -60,6 +60,29 @@ def test_silu_matvec_vs_f64(oracle, bits, gs, K, dtype_name, with_bias):
     assert _worst(y, _ref(o, *ops, dtype, gs, bits)) <= TOL
 
 
+@pytest.mark.parametrize("M", [2, 3, 4])
+@pytest.mark.parametrize("bits,dtype_name,K", [(8, "bf16", 3072), (4, "bf16", 3072), (8, "f16", 1024), (4, "f16", 4096)])
+def test_silu_matvec_up_to_four_rows(oracle, bits, dtype_name, K, M):
+    """Two to four activation rows (a batch): the activation inside the four-rows kernel."""
+    import mflux_amd
+    from gpu_util import to_dev
+
+    o = oracle
+    dtype = o.BF16 if dtype_name == "bf16" else o.F16
+    N = 1024 + 24
+    ops = _operands(o, 37, K, N, bits, 64, dtype, True)
+    xm = o._from_f32(seeded(37, 5, (M, K), 2.0) * np.float32([[1.0], [0.01], [30.0], [3.0]][:M]), dtype)
+    _, wq, s, b, bias = _dev(o, *ops, dtype)
+    y = mflux_amd.silu_quantized_matmul(to_dev(xm, dtype), wq, s, b, group_size=64, bits=bits, bias=bias)
+    torch.cuda.synchronize()
+    assert y.shape == (M, N)
+    ref = _ref(o, xm, *ops[1:], dtype, 64, bits)
+    assert _worst(y, ref) <= TOL
+    # and against the composition: the same kernel behind a separate activation
+    want = mflux_amd.quantized_matmul(mflux_amd.silu(to_dev(xm, dtype)), wq, s, b, group_size=64, bits=bits, bias=bias)
+    assert float((y.double() - want.double()).abs().max() / want.double().abs().max()) <= 2e-3
+
+
 def test_silu_matvec_adaln_full_size(oracle):
     """FLUX.1 double-block norm1: 3072 -> 18432, 8 bits, through the C ABI entry point itself."""
     from mflux_amd import _lib
@@ -69,7 +92,7 @@ def test_silu_matvec_adaln_full_size(oracle):
     ops = _operands(o, 32, K, N, 8, 64, o.BF16, True, x_std=1.0)
     x, wq, s, b, bias = _dev(o, *ops, o.BF16)
     y = torch.empty((1, N), dtype=torch.bfloat16, device="cuda")
-    rc = _lib.load().mfq_qmv_silu(x.data_ptr(), _lib.BF16, K, wq.data_ptr(), s.data_ptr(), b.data_ptr(), _lib.BF16,
+    rc = _lib.load().mfq_qmv_silu(x.data_ptr(), _lib.BF16, 1, K, wq.data_ptr(), s.data_ptr(), b.data_ptr(), _lib.BF16,
                                   bias.data_ptr(), N, 64, 8, y.data_ptr(), _lib.BF16,
                                   torch.cuda.current_stream().cuda_stream)
     assert rc == 0
@@ -125,12 +148,12 @@ def test_silu_fused_against_composition(oracle, bits):
 
 
 def test_silu_calls_without_a_fused_kernel_compose(oracle):
-    """More than one row, rows longer than the one-row kernel takes, odd bit
+    """More than four rows, rows longer than the fused kernels take, odd bit
     widths and float32 x run silu as its own pass: identical to the composition."""
     import mflux_amd
 
     o = oracle
-    for M, K, bits in ((4, 3072, 8), (1, 8192, 8), (1, 3072, 5), (3, 1024, 4)):
+    for M, K, bits in ((5, 3072, 8), (1, 8192, 8), (1, 3072, 5), (3, 8192, 4)):
         ops = _operands(o, 35, K, 256, bits, 64, o.BF16, True)
         x, wq, s, b, bias = _dev(o, *ops, o.BF16)
         x = x.expand(M, K).contiguous() * torch.arange(1, M + 1, device="cuda", dtype=torch.bfloat16)[:, None]
