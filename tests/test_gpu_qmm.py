@@ -729,7 +729,17 @@ def test_calls_replay_in_a_hip_graph(oracle):
         x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
         w = (torch.randn(N, K, device="cuda") * 0.02).to(torch.bfloat16)
         ops.append((x, *mflux_amd.quantize(w, 64, bits), bits))
-    run = lambda: [mflux_amd.quantized_matmul(x, wq, s, b, bits=bits) for x, wq, s, b, bits in ops]
+    x4 = torch.randn(4, 3072, device="cuda").to(torch.bfloat16)
+
+    def run():
+        outs = [mflux_amd.quantized_matmul(x, wq, s, b, bits=bits) for x, wq, s, b, bits in ops]
+        # the matvecs with the activation inside (one row, four rows) and the four-rows kernel as it is
+        x1, wq, s, b, bits = ops[0]
+        outs.append(mflux_amd.silu_quantized_matmul(x1, wq, s, b, bits=bits))
+        outs.append(mflux_amd.silu_quantized_matmul(x4, wq, s, b, bits=bits))
+        outs.append(mflux_amd.quantized_matmul(x4, wq, s, b, bits=bits))
+        return outs
+
     eager = run()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
