@@ -353,6 +353,15 @@ def main():
         gbs = nbytes / (ms * 1e-3) / 1e9
         quant[name] = {"us": round(ms * 1e3, 1), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
 
+    # the second half of the headline metric ("W8 GEMV GB/s at M=1") in the form of `roofline`: algorithmic
+    # bytes of one 3072 -> 18432 call over its time in a chain of graph launches; traffic from the committed
+    # FETCH_SIZE / WRITE_SIZE profile of the same kernel (62.7 MB read, 0.04 MB written)
+    gemv_roofline = None
+    if "w8" in gemv:
+        m1 = gemv["w8"]["M1"]
+        gemv_roofline = {"kernel": "qmv_dot_kernel<BF16,8,3>", "bound": "hbm", "achieved": m1["GB/s"],
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": m1["frac_hbm"], "traffic": 62.7e6 + 0.04e6,
+                         "avg_launch_us": m1["us"], "bytes_per_launch": m1["bytes"]}
     out = {
         "metric": "W4A16 qmatmul TFLOP/s @ FLUX single-block M=4608",
         "value": round(value, 2),
@@ -370,7 +379,8 @@ def main():
                    "M": M_TOKENS, "bits": BITS, "group_size": GS},
         "roofline": roofline,
         "per_shape": per_shape,
-        "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "gemv_w8": gemv.get("w8", {}),
+        "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "roofline": gemv_roofline,
+                      "gemv_w8": gemv.get("w8", {}),
                       "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
                       "qmm_w4_lora_r16": lora, "library_bf16_gemm_same_operands": library},
     }
