@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mfq.h"
 
 namespace mfq {
@@ -204,16 +206,56 @@ __device__ inline uint32_t silu_pair(uint32_t pair) {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Launch parameters that depend on the device (compute units, resident
+// workgroups of a kernel, "the LDS limit of this kernel has been raised") are
+// cached per device: a process may drive several GPUs, each from its own
+// threads.  A slot holds 0 until a thread has computed its value; two threads
+// that race compute the same value and store it twice.  Nothing is cached for a
+// device index outside the table.
+constexpr int kMaxDevices = 64;
+
+inline int device_index() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+  return dev;
+}
+
+struct PerDeviceInt {
+  std::atomic<int> slot[kMaxDevices];
+
+  // compute() returns the value (> 0) or a value <= 0 for "failed", which is
+  // handed back and not kept.
+  template <typename F>
+  int get(F compute) {
+    const int dev = device_index();
+    if (dev < 0) return compute();
+    int v = slot[dev].load(std::memory_order_acquire);
+    if (v == 0) {
+      v = compute();
+      if (v > 0) slot[dev].store(v, std::memory_order_release);
+    }
+    return v;
+  }
+};
+
 // Compute units of the current device (256 on an MI355X).
 inline int compute_units() {
-  static int n = 0;
-  if (n == 0) {
+  static PerDeviceInt cache;
+  const int n = cache.get([] {
     int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
-    n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  }
-  return n;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+    return prop.multiProcessorCount;
+  });
+  return n > 0 ? n : 256;
+}
+
+// Raises a kernel's dynamic LDS limit once per device; `done` is the launcher's
+// own static cache (one per kernel instantiation).
+inline bool raise_lds_limit(PerDeviceInt& done, const void* kernel, int bytes) {
+  return done.get([&] {
+           return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess ? 1 : -1;
+         }) > 0;
 }
 
 // A low-rank update added to a product, y += t @ bs^T: t [M, R] holds the

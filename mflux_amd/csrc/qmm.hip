@@ -886,13 +886,8 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
                   const void* bias, int64_t N, void* y, int y_dtype, TailPlan plan, void* planes, hipStream_t stream,
                   LowRank lr = LowRank()) {
   auto kernel = qmm_kernel<T, GS, BITS, kFast, kLowRank>;
-  static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLdsBytes) != hipSuccess)
-      return MFQ_ELAUNCH;
-    configured = true;
-  }
+  static PerDeviceInt configured;
+  if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
   const int n_tail = tiles_m * tiles_n - plan.n_whole;

@@ -451,13 +451,8 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
                   const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr) {
   auto kernel = qmm_mid_kernel<T, GS, BITS, kFast, kWavesM>;
   constexpr int kLds = lds_bytes(kWavesM);
-  static bool configured = false;  // raising the dynamic LDS limit is a per-function, per-process setting
-  if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kLds) != hipSuccess)
-      return MFQ_ELAUNCH;
-    configured = true;
-  }
+  static PerDeviceInt configured;
+  if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLds)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + tile_m(kWavesM) - 1) / tile_m(kWavesM));
   const int tiles_n = (int)((N + TN - 1) / TN);
   const int64_t n_items = (int64_t)tiles_m * tiles_n * plan.splits;

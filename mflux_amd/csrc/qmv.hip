@@ -464,12 +464,12 @@ int launch_rows_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, 
   // as many workgroups as are resident at once (the register count of the
   // instantiation decides), so that every wavefront gets one balanced run of rows
   auto kernel = qmv_rows_kernel<T, BITS, kM, kMaxLoads, kCoop>;
-  static int blocks_per_cu = 0;
-  if (blocks_per_cu == 0) {
+  static PerDeviceInt cache;
+  const int blocks_per_cu = cache.get([&] {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) n = 1;
-    blocks_per_cu = n > 4 ? 4 : n;
-  }
+    return n > 4 ? 4 : n;
+  });
   int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
   const int64_t max_blocks = (N + 3) / 4;  // at least one row per wavefront
   if (blocks > max_blocks) blocks = max_blocks;
@@ -550,14 +550,10 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   using P = Phase<T, GS, BITS>;
   auto kernel = qmv_kernel<T, GS, BITS>;
   const size_t lds_bytes = 2 * ((size_t)P::kXTileOffset + (size_t)M * P::kRowBytes);
-  static bool configured = false;
-  if (!configured) {
-    // largest request: M = 16 rows of a 4-bit phase (2048 k), double buffered, about 140 KiB
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * (P::kXTileOffset + 16 * P::kRowBytes)) != hipSuccess)
-      return MFQ_ELAUNCH;
-    configured = true;
-  }
+  // largest request: M = 16 rows of a 4-bit phase (2048 k), double buffered, about 140 KiB
+  static PerDeviceInt configured;
+  if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), 2 * (P::kXTileOffset + 16 * P::kRowBytes)))
+    return MFQ_ELAUNCH;
   const dim3 grid((unsigned)((N + kRowsPerBlock - 1) / kRowsPerBlock));
   hipLaunchKernelGGL(kernel, grid, dim3(256), lds_bytes, stream, (const uint16_t*)x, wq, (const uint16_t*)scales,
                      (const uint16_t*)biases, (const uint16_t*)bias, y, (int)(y_dtype == MFQ_F32), (int)M, (int)N,

@@ -337,12 +337,12 @@ int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scal
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
   auto kernel = qmv_dot_kernel<T, BITS, kLoads, kCoop, kSilu>;
   const size_t lds = (size_t)(K * BITS / 8 / 16) * (BITS == 8 ? 8 : 16) * 4;  // the x image: 2 bytes per element
-  static int resident = 0;  // workgroups of this instantiation a compute unit holds
-  if (resident == 0) {
+  static PerDeviceInt cache;  // workgroups of this instantiation a compute unit holds
+  const int resident = cache.get([&] {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, lds) != hipSuccess || n < 1) n = 1;
-    resident = n > 4 ? 4 : n;
-  }
+    return n > 4 ? 4 : n;
+  });
   // Workgroups per compute unit: enough wavefronts for about 48 KiB of weight rows in flight (two
   // rows each), not more: every workgroup pays for its own image of x.  Measured at K = 3072: two
   // workgroups for 3 KiB rows (W8), four for 1.5 KiB rows (W4).  One fewer when that deals the rows

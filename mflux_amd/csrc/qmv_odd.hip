@@ -237,12 +237,12 @@ template <typename T, int BITS, int kUnits>
 int launch_kernel(const void* x, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                   const void* bias, int64_t N, int gs_shift, void* y, int y_dtype, hipStream_t stream) {
   auto kernel = qmv_odd_kernel<T, BITS, kUnits>;
-  static int blocks_per_cu = 0;
-  if (blocks_per_cu == 0) {
+  static PerDeviceInt cache;
+  const int blocks_per_cu = cache.get([&] {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) n = 1;
-    blocks_per_cu = n > 4 ? 4 : n;
-  }
+    return n > 4 ? 4 : n;
+  });
   // as many workgroups as are resident at once, so that every wavefront gets one balanced run of rows
   int64_t blocks = (int64_t)compute_units() * blocks_per_cu;
   const int64_t max_blocks = (N + 3) / 4;

@@ -338,18 +338,19 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   auto kernel = qmv_quad_kernel<T, BITS, kLoads, kRing, kSilu>;
   constexpr int kXOps = 128 / BITS / 4;
   constexpr int kLds = kLoads * kXOps * 512 + kLoads * 256 + 4 * 2 * kScaleRegion + 64;  // + the rows' largest magnitudes
-  static int blocks_per_cu = 0;
-  if (blocks_per_cu == 0) {
+  static PerDeviceInt cache;
+  const int blocks_per_cu = cache.get([&] {
     if (kLds > 48 * 1024 &&
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) !=
             hipSuccess)
-      return MFQ_ELAUNCH;
+      return -1;
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, kLds) != hipSuccess || n < 1) n = 1;
     // two workgroups per compute unit: every workgroup stages x for itself, and more of them measured
     // slower (3072 -> 18432 at M = 4: 17.8 us with two, 19.0 us with three or four)
-    blocks_per_cu = n > 2 ? 2 : n;
-  }
+    return n > 2 ? 2 : n;
+  });
+  if (blocks_per_cu < 1) return MFQ_ELAUNCH;
   // At most that many wavefronts, and every one of them the same number of
   // quads: with 4608 quads, 1536 wavefronts of three finish together, whereas
   // 2048 wavefronts would leave 512 of them a third quad.
