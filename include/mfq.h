@@ -50,7 +50,9 @@ enum mfq_status {
   MFQ_ENULL = -5,      /* a required pointer is NULL                         */
   MFQ_EALIGN = -6,     /* a buffer is not 16-byte aligned                    */
   MFQ_ELAUNCH = -7,    /* the HIP runtime refused the launch                 */
-  MFQ_EUNSUPPORTED = -8 /* valid request that this build has no kernel for   */
+  MFQ_EUNSUPPORTED = -8, /* valid request that this build has no kernel for  */
+  MFQ_ESCRATCH = -9     /* mfq_qmm_t_static: the shape's K split needs more
+                           than MFQ_STATIC_SCRATCH_BYTES                      */
 };
 
 /* Library version: major*10000 + minor*100 + patch. */
@@ -158,6 +160,29 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  const void* scales, const void* biases, int sb_dtype, const void* bias, int64_t N,
                  int group_size, int bits, void* y, int y_dtype, void* workspace,
                  size_t workspace_bytes, void* stream);
+
+/*
+ * mfq_qmm_t_ws for callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  Has no counterpart in
+ * the reference.  The float32 planes of the K split live in a buffer of
+ * MFQ_STATIC_SCRATCH_BYTES that is part of the library's device image (every
+ * GPU the library runs on holds its own copy until the process ends), so the
+ * call allocates nothing and takes no workspace: same arguments as mfq_qmm_t,
+ * same kernels and bit-identical results as mfq_qmm_t_ws with a workspace of
+ * mfq_qmm_t_workspace_bytes().  A shape whose split needs more than the
+ * buffer holds is refused with MFQ_ESCRATCH and nothing is launched (on a
+ * 256-CU device: the last, short round of 256 x 256 tiles cut into more than
+ * 128 planes, e.g. M = 6889 against 3072 -> 3072; use mfq_qmm_t_ws or
+ * mfq_qmm_t there).  All calls on one GPU share that GPU's buffer: calls that
+ * overlap on one GPU (two streams, two threads) race; order them on one
+ * stream.  The buffer's contents between calls are undefined; nothing in it
+ * has to be zero.  The first call on a device looks the buffer's address up
+ * and configures the kernels; make it outside a graph capture.
+ */
+#define MFQ_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int mfq_qmm_t_static(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
+                     const void* scales, const void* biases, int sb_dtype, const void* bias,
+                     int64_t N, int group_size, int bits, void* y, int y_dtype, void* stream);
 
 /*
  * y[m, n] = sum_k silu(x)[m, k] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs]) (+ bias[n]):

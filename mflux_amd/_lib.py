@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmfq.so")
 
 F32, F16, BF16 = 0, 1, 2
 MFQ_EUNSUPPORTED = -8  # no kernel for this combination of arguments
+MFQ_ESCRATCH = -9  # mfq_qmm_t_static: the K split needs more than the built-in buffer
 
 # every symbol include/mfq.h declares, with its ctypes signature
 _I64, _INT, _PTR = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p
@@ -26,6 +27,7 @@ SIGNATURES = {
     "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,
                             ctypes.c_size_t, _PTR]),
+    "mfq_qmm_t_static": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t_low_rank": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _PTR,
                                   _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),
     "mfq_qmv_silu": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),

@@ -14,6 +14,27 @@ int check_common(int gs, int bits) {
 bool is16(int dtype) { return dtype == MFQ_BF16 || dtype == MFQ_F16; }
 bool known(int dtype) { return dtype == MFQ_F32 || is16(dtype); }
 
+// The float32 planes of mfq_qmm_t_static's K split.  Every device the library
+// runs on holds its own copy of this array, at its own address, until the
+// process ends; the name below is only the host's handle for it, the address
+// on the current device comes from hipGetSymbolAddress (scratch_on_device).
+constexpr size_t kScratchBytes = MFQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+std::atomic<void*> scratch_ptr[mfq::kMaxDevices];
+
+// Address of `scratch` on the current device, looked up once per device.
+int scratch_on_device(void** out) {
+  const int dev = mfq::device_index();
+  if (dev < 0) return MFQ_ELAUNCH;
+  void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MFQ_ELAUNCH;
+    scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return MFQ_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -31,6 +52,7 @@ const char* mfq_strerror(int status) {
     case MFQ_EALIGN: return "buffers must be 16-byte aligned";
     case MFQ_ELAUNCH: return "HIP launch failed";
     case MFQ_EUNSUPPORTED: return "no kernel for this combination";
+    case MFQ_ESCRATCH: return "the shape needs more scratch than the library's built-in buffer holds";
     default: return "unknown status";
   }
 }
@@ -87,6 +109,20 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  int y_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   return mfq_qmm_t_low_rank(x, x_dtype, M, K, wq, scales, biases, sb_dtype, bias, N, group_size, bits, nullptr, nullptr,
                             0, y, y_dtype, workspace, workspace_bytes, stream);
+}
+
+int mfq_qmm_t_static(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                     const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
+                     int y_dtype, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  const size_t need = mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits);
+  if (need > kScratchBytes) return MFQ_ESCRATCH;
+  void* ws = nullptr;
+  if (need) {
+    if (int rc = scratch_on_device(&ws)) return rc;
+  }
+  return mfq_qmm_t_low_rank(x, x_dtype, M, K, wq, scales, biases, sb_dtype, bias, N, group_size, bits, nullptr, nullptr,
+                            0, y, y_dtype, ws, need, stream);
 }
 
 int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
