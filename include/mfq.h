@@ -24,10 +24,8 @@
  *     word i / (32/bits); for 3, 5 and 6 bits it is MLX's 3- and 5-byte packs
  *     laid end to end.  scales and biases hold one value per `group_size`
  *     consecutive elements of a row.
- *   - bits: 3, 4, 5, 6, 8 for quantize / dequantize / dequantize_rows (3, 5, 6
- *     for 16-bit inputs only); 4 and 8 for qmm_t, and 3, 5, 6 for qmm_t with
- *     one activation row and K <= 8192 (MFQ_EUNSUPPORTED otherwise:
- *     dequantize and use a plain GEMM).
+ *   - bits: 3, 4, 5, 6, 8 everywhere (quantize of 3, 5, 6 bits takes 16-bit
+ *     inputs only).
  */
 #ifndef MFQ_H
 #define MFQ_H
@@ -66,7 +64,10 @@ const char* mfq_strerror(int status);
  * Replaces mx.quantize(w, group_size, bits, mode="affine") as reached from
  * nn.quantize at src/mflux/models/common/weights/loading/
  * weight_applier.py:43,46,103 (Linear.to_quantized -> QuantizedLinear.
- * from_linear).  Results are bit-identical to MLX's CPU evaluation.
+ * from_linear).  Results are bit-identical to oracle/mlx_affine.c, a
+ * restatement of MLX's CPU algorithm (quantize<T,U>); parity with MLX itself
+ * is unpinned: MLX cannot be run where this library is built and the
+ * reference holds no vector for this function.
  *   w       [rows, K]              dtype
  *   wq      [rows, K*bits/32]      uint32
  *   scales  [rows, K/group_size]   dtype
@@ -80,7 +81,12 @@ int mfq_quantize_affine(const void* w, int dtype, int64_t rows, int64_t K,
  * Inverse mapping w = code*scale + bias, written in `out_dtype`.
  * Replaces mx.dequantize; mflux needs it where a LoRA is baked into a
  * quantized base (src/mflux/models/common/lora/mapping/lora_saver.py:59-82).
- * The value is the float32 fma(code, scale, bias) rounded once to out_dtype.
+ * mx.dequantize is an element-wise multiply followed by an element-wise add
+ * on arrays of the output type: the product code * scale is rounded to
+ * out_dtype, then the sum with the bias is rounded to out_dtype (for float32
+ * output from 16-bit scales both steps are exact up to the one final
+ * rounding).  Bit-identical to mlxo_dequantize of oracle/mlx_affine.c; parity
+ * with MLX itself is unpinned.
  */
 int mfq_dequantize_affine(const uint32_t* wq, const void* scales,
                           const void* biases, int sb_dtype, int64_t rows,
@@ -124,7 +130,9 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
  *   y       [M, N]                 y_dtype (sb_dtype or MFQ_F32)
  * M <= 16 runs the HBM-bound dequant-GEMV kernel, larger M one of two MFMA
  * GEMM kernels (128-column tiles while 256 x 256 tiles would leave more than
- * half of the compute units idle, 256 x 256 tiles otherwise).  For M > 4 the
+ * half of the compute units idle, 256 x 256 tiles otherwise).  3, 5 and 6 bits:
+ * one activation row of up to 8192 elements has its own kernel, everything
+ * else runs on the 128-column-tile GEMM.  For M > 4 the
  * dequantised weights are rounded once to x_dtype and sums are float32.  For
  * M <= 4 (4 and 8 bits; shapes the integer kernels take) every row of x
  * becomes 15-bit fixed point (one power of two per row brings its largest
@@ -137,6 +145,26 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
               const uint32_t* wq, const void* scales, const void* biases,
               int sb_dtype, const void* bias, int64_t N, int group_size,
               int bits, void* y, int y_dtype, void* stream);
+
+/*
+ * y[m, k] = sum_n x[m, n] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs]):
+ * the product with the weight NOT transposed.  Replaces
+ * mx.quantized_matmul(x, w, scales, biases, transpose=False, ...), which is the
+ * gradient of a quantized linear with respect to its input: MLX's autograd
+ * evaluates it for every QuantizedLinear that
+ * src/mflux/models/common/training/lora/target_injector.py:30-33 wraps in a
+ * trainable LoRALinear.
+ *   x       [M, N]                 x_dtype (MFQ_BF16 or MFQ_F16; must equal sb_dtype)
+ *   wq      [N, K*bits/32]         uint32
+ *   scales, biases [N, K/group_size]   sb_dtype
+ *   y       [M, K]                 y_dtype (sb_dtype or MFQ_F32)
+ * Dequantised weights are rounded once to x_dtype, sums are float32.
+ * MFQ_EUNSUPPORTED when N is not a multiple of 8 (pad x with zero columns and
+ * the packed weight, scales and biases with as many rows).
+ */
+int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+              const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y,
+              int y_dtype, void* stream);
 
 /*
  * mfq_qmm_t with an optional float32 workspace.  Has no counterpart in the

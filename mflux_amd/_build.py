@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libmfq.so")
-SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmm.hip", "qmm_mid.hip", "lora.hip")
+SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmm.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "lora.hip")
 
 # -ffp-contract=off, correctly rounded division and preserved denormals make
 # the quantize kernel's float32 arithmetic the same IEEE operations as the
@@ -57,5 +57,30 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+OPS_PATH = os.path.join(CSRC, "libmfq_torch.so")
+
+
+def build_torch_ops(verbose: bool = False) -> str:
+    """Compiles csrc/torch_ops.cpp (the torch.ops.mfq registrations, host C++
+    only) against this interpreter's torch and links it to libmfq.so."""
+    from torch.utils import cpp_extension
+
+    torch_lib = cpp_extension.library_paths()[0]
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    tmp = OPS_PATH + ".tmp"
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=1", *[f"-I{p}" for p in cpp_extension.include_paths()], f"-I{rocm}/include",
+           os.path.join(CSRC, "torch_ops.cpp"), "-o", tmp, f"-L{CSRC}", "-lmfq", f"-L{torch_lib}", "-ltorch",
+           "-ltorch_cpu", "-lc10", "-ltorch_hip", "-lc10_hip", "-Wl,-rpath,$ORIGIN"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"g++ failed on torch_ops.cpp:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, OPS_PATH)
+    if verbose:
+        print(f"built {OPS_PATH}")
+    return OPS_PATH
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
+    build_torch_ops(verbose=True)

@@ -24,6 +24,7 @@ SIGNATURES = {
     "mfq_dequantize_affine": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_dequantize_rows": (_INT, [_PTR, _PTR, _PTR, _INT, _PTR, _I64, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmm_n": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,
                             ctypes.c_size_t, _PTR]),
@@ -61,6 +62,25 @@ def load() -> ctypes.CDLL:
             fn.argtypes = argtypes
         _lib = lib
     return _lib
+
+
+OPS_PATH = os.path.join(_HERE, "csrc", "libmfq_torch.so")
+_ops = None
+
+
+def ops():
+    """``torch.ops.mfq``: the ops of csrc/torch_ops.cpp over the same libmfq.so
+    (its RUNPATH is its own directory).  Raises if either library is not built."""
+    global _ops
+    if _ops is None:
+        import torch
+
+        load()
+        if not os.path.exists(OPS_PATH):
+            raise ImportError(f"{OPS_PATH} is missing: build it with `python -m mflux_amd._build`")
+        torch.ops.load_library(OPS_PATH)
+        _ops = torch.ops.mfq
+    return _ops
 
 
 def check(fn: str, status: int) -> None:

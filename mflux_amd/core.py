@@ -8,7 +8,9 @@ quantized ``nn.Linear`` call such as
 src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53,57.
 
 Tensors are torch tensors on a HIP device; torch only provides the device
-memory and the stream, the arithmetic is libmfq's hand-written kernels.
+memory and the stream, the arithmetic is libmfq's hand-written kernels, reached
+through the ``torch.ops.mfq`` ops of csrc/torch_ops.cpp (a thin C++ layer over
+the C ABI of include/mfq.h).
 """
 from __future__ import annotations
 
@@ -20,11 +22,7 @@ _DTYPE_CODE = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16:
 SUPPORTED_GROUP_SIZES = (32, 64, 128)
 MLX_BITS = (2, 3, 4, 5, 6, 8)  # what mx.quantize accepts
 SUPPORTED_BITS = (3, 4, 5, 6, 8)  # what quantize / dequantize have kernels for
-MATMUL_KERNEL_BITS = (4, 8)  # what the matvec / GEMM kernels unpack themselves
-
-
-def _stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+MATMUL_KERNEL_BITS = (4, 8)  # what the SiLU-fused matvec kernels take
 
 
 def _check_mode(fn: str, mode: str) -> None:
@@ -60,7 +58,9 @@ def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4, mode: str = "
 
     Returns ``(w_q, scales, biases)``: ``w_q`` uint32 ``[..., K*bits/32]`` with
     element ``i`` of each word at bit offset ``i*bits``; ``scales``/``biases`` of
-    ``w``'s dtype, ``[..., K/group_size]``.  Bit-identical to MLX's CPU result.
+    ``w``'s dtype, ``[..., K/group_size]``.  Bit-identical to the restatement of
+    MLX's CPU algorithm in oracle/mlx_affine.c (parity with MLX itself is
+    unpinned: it cannot be run here).
     """
     _check_mode("quantize", mode)
     _check_group_bits("quantize", group_size, bits)
@@ -80,19 +80,9 @@ def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4, mode: str = "
         raise NotImplementedError(f"[quantize] {bits}-bit quantization of float32 input is not implemented in "
                                   "this build; cast to bfloat16 or float16")
     _require_hip("quantize", w, "w")
-    w = w.contiguous()
     lead = tuple(w.shape[:-1])
-    rows = w.numel() // K
-    wq = torch.empty((*lead, K * bits // 32), dtype=torch.uint32, device=w.device)
-    scales = torch.empty((*lead, K // group_size), dtype=w.dtype, device=w.device)
-    biases = torch.empty_like(scales)
-    with torch.cuda.device(w.device):
-        rc = _lib.load().mfq_quantize_affine(
-            w.data_ptr(), _DTYPE_CODE[w.dtype], rows, K, group_size, bits,
-            wq.data_ptr(), scales.data_ptr(), biases.data_ptr(), _stream_ptr(w.device),
-        )
-    _lib.check("mfq_quantize_affine", rc)
-    return wq, scales, biases
+    wq, scales, biases = _lib.ops().quantize_affine(w.reshape(-1, K).contiguous(), group_size, bits)
+    return wq.reshape(*lead, -1), scales.reshape(*lead, -1), biases.reshape(*lead, -1)
 
 
 def _check_packed(fn: str, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int, bits: int):
@@ -115,10 +105,15 @@ def _check_packed(fn: str, w: torch.Tensor, scales: torch.Tensor, biases: torch.
         )
 
 
+def _rows2d(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape(-1, t.shape[-1]).contiguous()
+
+
 def dequantize(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64, bits: int = 4,
                mode: str = "affine", dtype: torch.dtype | None = None) -> torch.Tensor:
-    """``code * scale + bias`` in ``dtype`` (default: the dtype of ``scales``).
-    The value is the float32 fused multiply-add rounded once."""
+    """``code * scale + bias`` in ``dtype`` (default: the dtype of ``scales``),
+    evaluated as ``mx.dequantize`` does: the product is rounded to ``dtype``, then
+    the sum is."""
     _check_mode("dequantize", mode)
     _check_group_bits("dequantize", group_size, bits)
     _check_packed("dequantize", w, scales, biases, group_size, bits)
@@ -126,17 +121,9 @@ def dequantize(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, grou
     out_dtype = scales.dtype if dtype is None else dtype
     if out_dtype not in (scales.dtype, torch.float32):
         raise ValueError(f"[dequantize] Output dtype must be {scales.dtype} or float32, got {out_dtype}")
-    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
     K = w.shape[-1] * 32 // bits
-    rows = w.numel() // w.shape[-1]
-    out = torch.empty((*w.shape[:-1], K), dtype=out_dtype, device=w.device)
-    with torch.cuda.device(w.device):
-        rc = _lib.load().mfq_dequantize_affine(
-            w.data_ptr(), scales.data_ptr(), biases.data_ptr(), _DTYPE_CODE[scales.dtype], rows, K, group_size, bits,
-            out.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(w.device),
-        )
-    _lib.check("mfq_dequantize_affine", rc)
-    return out
+    out = _lib.ops().dequantize_affine(_rows2d(w), _rows2d(scales), _rows2d(biases), group_size, bits, out_dtype)
+    return out.reshape(*w.shape[:-1], K)
 
 
 def dequantize_rows(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, indices: torch.Tensor,
@@ -159,16 +146,8 @@ def dequantize_rows(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
         raise ValueError(f"[dequantize] Output dtype must be {scales.dtype} or float32, got {out_dtype}")
     K = w.shape[1] * 32 // bits
     idx = indices.to(device=w.device, dtype=torch.int64).reshape(-1).contiguous()
-    out = torch.empty((idx.numel(), K), dtype=out_dtype, device=w.device)
-    if idx.numel() == 0:
-        return out.reshape(*indices.shape, K)
-    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
-    with torch.cuda.device(w.device):
-        rc = _lib.load().mfq_dequantize_rows(
-            w.data_ptr(), scales.data_ptr(), biases.data_ptr(), _DTYPE_CODE[scales.dtype], idx.data_ptr(), idx.numel(),
-            w.shape[0], K, group_size, bits, out.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(w.device),
-        )
-    _lib.check("mfq_dequantize_rows", rc)
+    out = _lib.ops().dequantize_rows(w.contiguous(), scales.contiguous(), biases.contiguous(), idx, group_size, bits,
+                                     out_dtype)
     return out.reshape(*indices.shape, K)
 
 
@@ -177,11 +156,15 @@ def _matmul_untransposed(x, w, scales, biases, group_size, bits):
     product MLX computes for ``transpose=False``, which is what the gradient of a
     quantized linear with respect to its input needs when a LoRA is trained on a
     quantized base (src/mflux/models/common/training/lora/target_injector.py:30-33
-    wraps ``nn.QuantizedLinear`` in a trainable ``LoRALinear``).  Composed
-    from this library's dequantize kernel and the BLAS library's GEMM."""
+    wraps ``nn.QuantizedLinear`` in a trainable ``LoRALinear``).  One kernel
+    (``mfq_qmm_n``): the weight tile is dequantised and transposed on its way
+    into LDS; float32 ``x`` is rounded to the dtype of ``scales`` as for
+    ``transpose=True``."""
     _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
     if w.ndim != 2:
         raise NotImplementedError("[quantized_matmul] batched weights are not implemented in this build")
+    if scales.dtype == torch.float32:
+        raise NotImplementedError("[quantized_matmul] float32 scales are not implemented in this build")
     N = w.shape[0]
     K = w.shape[1] * 32 // bits
     if x.ndim < 1 or x.shape[-1] != N:
@@ -191,11 +174,25 @@ def _matmul_untransposed(x, w, scales, biases, group_size, bits):
             f"group_size={group_size}, bits={bits} and transpose=false"
         )
     _require_hip("quantized_matmul", x, "x")
+    _require_hip("quantized_matmul", w, "w")
     out_dtype = torch.result_type(x, scales)
-    w_full = dequantize(w, scales, biases, group_size, bits)
-    if out_dtype == scales.dtype:
-        return torch.matmul(x.to(scales.dtype), w_full)
-    return torch.matmul(x.float(), w_full.float())
+    lead = tuple(x.shape[:-1])
+    x2 = x.reshape(-1, N).to(scales.dtype)
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    if N % 8:
+        # the kernel reads x in 16-byte pieces: zero columns of x against zero rows of the weight add nothing
+        pad = 8 - N % 8
+        x2 = torch.nn.functional.pad(x2, (0, pad))
+        w = torch.cat([w, w.new_zeros((pad, w.shape[1]))])
+        scales = torch.cat([scales, scales.new_zeros((pad, scales.shape[1]))])
+        biases = torch.cat([biases, biases.new_zeros((pad, biases.shape[1]))])
+    if x2.shape[0] == 0:
+        return torch.empty((*lead, K), dtype=out_dtype, device=x.device)
+    y, ok = _lib.ops().qmm_n(x2.contiguous(), w, scales, biases, group_size, bits, out_dtype)
+    if not ok:
+        raise NotImplementedError(f"[quantized_matmul] no kernel for x {tuple(x.shape)} against a weight of "
+                                  f"{N} x {K} with transpose=False (an operand exceeds 2 GiB)")
+    return y.reshape(*lead, K)
 
 
 class _QuantizedMatmulFunction(torch.autograd.Function):
@@ -281,16 +278,9 @@ def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor
             if bias.shape != (N,):
                 raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
             bias = bias.to(x.dtype).contiguous()
-        x1 = x.reshape(M, K).contiguous()
-        w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
-        y = torch.empty((M, N), dtype=x.dtype, device=x.device)
-        with torch.cuda.device(x.device):
-            rc = _lib.load().mfq_qmv_silu(
-                x1.data_ptr(), _DTYPE_CODE[x.dtype], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
-                _DTYPE_CODE[x.dtype], bias.data_ptr() if bias is not None else None, N, group_size, bits,
-                y.data_ptr(), _DTYPE_CODE[x.dtype], _stream_ptr(x.device))
-        if rc != _lib.MFQ_EUNSUPPORTED:
-            _lib.check("mfq_qmv_silu", rc)
+        y, ok = _lib.ops().qmv_silu(x.reshape(M, K).contiguous(), w.contiguous(), scales.contiguous(),
+                                    biases.contiguous(), bias, group_size, bits)
+        if ok:
             return y.reshape(*x.shape[:-1], N)
     return quantized_matmul(silu(x), w, scales, biases, transpose=True, group_size=group_size, bits=bits, mode=mode,
                             bias=bias)
@@ -357,59 +347,19 @@ def _quantized_matmul_forward(x: torch.Tensor, w: torch.Tensor, scales: torch.Te
         x2 = x2.to(compute)
     x2 = x2.contiguous()
     M = x2.shape[0]
-    y = torch.empty((M, N), dtype=out_dtype, device=x.device)
     if M == 0:
-        return y.reshape(*lead, N)
+        return torch.empty((*lead, N), dtype=out_dtype, device=x.device)
     if bias is not None:
         if bias.shape != (N,):
             raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
         bias = bias.to(compute).contiguous()
     w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
-    lib = _lib.load()
+    ops = _lib.ops()
     lr_t = lr_bs = None
-    rank = 0
     if low_rank is not None:
-        lr_t, lr_bs, rank = _low_rank_operands(low_rank, lead, M, N, compute)
-    if bits not in MATMUL_KERNEL_BITS:
-        # 3, 5 and 6 bits.  One activation row (the adaLN modulation calls) has a
-        # fused kernel; anything else, or a shape that kernel does not take, is
-        # this library's dequantize kernel (same single rounding as inside the
-        # fused kernels) followed by the BLAS library's plain GEMM, float32
-        # accumulation, the bias added after rounding y.
-        if M == 1:
-            with torch.cuda.device(x.device):
-                rc = lib.mfq_qmm_t_low_rank(
-                    x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
-                    _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
-                    lr_t.data_ptr() if rank else None, lr_bs.data_ptr() if rank else None, rank,
-                    y.data_ptr(), _DTYPE_CODE[out_dtype], None, 0, _stream_ptr(x.device),
-                )
-            if rc != _lib.MFQ_EUNSUPPORTED:
-                _lib.check("mfq_qmm_t_low_rank", rc)
-                return y.reshape(*lead, N)
-        w_full = dequantize(w, scales, biases, group_size, bits)
-        y = torch.matmul(x2, w_full.t()) if out_dtype == compute else torch.matmul(x2.float(), w_full.float().t())
-        if bias is not None:
-            y = y + bias.to(y.dtype)
-        if rank:
-            y = y.contiguous()
-            with torch.cuda.device(x.device):
-                rc = lib.mfq_low_rank_add(lr_t.data_ptr(), lr_bs.data_ptr(), _DTYPE_CODE[compute], M, N, rank,
-                                          y.data_ptr(), _DTYPE_CODE[out_dtype], _stream_ptr(x.device))
-            _lib.check("mfq_low_rank_add", rc)
-        return y.reshape(*lead, N)
-    with torch.cuda.device(x.device):
-        # few output tiles (text-stream shapes): K is split across compute units
-        # through a float32 scratch, taken from torch's caching allocator on the
-        # current stream (so its reuse is ordered after this call)
-        ws_bytes = lib.mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits)
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
-        rc = lib.mfq_qmm_t_low_rank(
-            x2.data_ptr(), _DTYPE_CODE[compute], M, K, w.data_ptr(), scales.data_ptr(), biases.data_ptr(),
-            _DTYPE_CODE[compute], bias.data_ptr() if bias is not None else None, N, group_size, bits,
-            lr_t.data_ptr() if rank else None, lr_bs.data_ptr() if rank else None, rank,
-            y.data_ptr(), _DTYPE_CODE[out_dtype], ws.data_ptr() if ws is not None else None, ws_bytes,
-            _stream_ptr(x.device),
-        )
-    _lib.check("mfq_qmm_t_low_rank", rc)
+        lr_t, lr_bs, _ = _low_rank_operands(low_rank, lead, M, N, compute)
+    y, ok = ops.qmm_t(x2, w, scales, biases, bias, group_size, bits, out_dtype, lr_t, lr_bs)
+    if not ok:
+        raise NotImplementedError(f"[quantized_matmul] no kernel for x {tuple(x.shape)} against a weight of "
+                                  f"{N} x {K} (an operand exceeds 2 GiB: split the rows of x)")
     return y.reshape(*lead, N)

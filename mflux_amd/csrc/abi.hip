@@ -92,8 +92,10 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
 }
 
 size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits) {
-  if (check_common(group_size, bits) != MFQ_OK || (bits != 4 && bits != 8)) return 0;
-  if (M <= 16 || N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  if (check_common(group_size, bits) != MFQ_OK) return 0;
+  if (N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  if (bits != 4 && bits != 8) return M > 1 ? mfq::qmm_mid_workspace_bytes(M, N, K, group_size) : 0;
+  if (M <= 16) return 0;
   return mfq::qmm_workspace_bytes(M, N, K, group_size);
 }
 
@@ -139,9 +141,7 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
     low_rank.bs = bs;
     low_rank.R = (int)rank;
   }
-  // 3, 5, 6 bits: a fused kernel for one activation row only; otherwise the caller dequantizes and uses a plain GEMM
   const bool odd_bits = bits != 4 && bits != 8;
-  if (odd_bits && M != 1) return MFQ_EUNSUPPORTED;
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
   if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
   if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
@@ -150,30 +150,39 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
   if (!mfq::aligned16(x) || !mfq::aligned16(wq)) return MFQ_EALIGN;
   if (M > 16 && !mfq::aligned16(y)) return MFQ_EALIGN;  // the GEMM writes y in 16-byte pieces
   if (odd_bits) {
-    const int rc = mfq::launch_qmv_odd(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
-                                       (hipStream_t)stream);
-    return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
+    // 3, 5, 6 bits: the one-row kernel for the rows it takes, the 128-column-tile GEMM for everything else
+    if (M == 1) {
+      const int rc = mfq::launch_qmv_odd(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                         (hipStream_t)stream);
+      if (rc != MFQ_EUNSUPPORTED)
+        return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
+    }
+    if (!mfq::aligned16(y)) return MFQ_EALIGN;
+    return mfq::launch_qmm_mid_stream(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                      workspace, workspace_bytes, (hipStream_t)stream, low_rank);
   }
   if (M <= 16) {
     const int rc = mfq::launch_qmv(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                                    (hipStream_t)stream);
     return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
   }
-  if (K % 64) {
-    // group size 32 with K an odd multiple of it: the matrix-core GEMM steps k
-    // by 64, so these rare shapes go through the small-M kernel 16 rows at a time
-    const size_t x_row = (size_t)K * 2, y_row = (size_t)N * (y_dtype == MFQ_F32 ? 4 : 2);
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
-      const int64_t rows = M - m0 < 16 ? M - m0 : 16;
-      const int rc = mfq::launch_qmv(static_cast<const char*>(x) + m0 * x_row, x_dtype, rows, K, wq, scales, biases,
-                                     bias, N, group_size, bits, static_cast<char*>(y) + m0 * y_row, y_dtype,
-                                     (hipStream_t)stream);
-      if (rc) return rc;
-    }
-    return mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
-  }
+  if (K % 64)  // group size 32 with K an odd multiple of it: the 128-column-tile GEMM pads the last k step with zeros
+    return mfq::launch_qmm_mid(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, nullptr, 0,
+                               (hipStream_t)stream, low_rank);
   return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, workspace,
                          workspace_bytes, (hipStream_t)stream, low_rank);
+}
+
+int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+              const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y, int y_dtype, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
+  if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
+  if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || N * (K * bits / 32) >= (int64_t)1 << 31) return MFQ_ESHAPE;
+  if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
+  if (!mfq::aligned16(x) || !mfq::aligned16(wq) || !mfq::aligned16(y)) return MFQ_EALIGN;
+  return mfq::launch_qmm_n(x, x_dtype, M, N, wq, scales, biases, K, group_size, bits, y, y_dtype, (hipStream_t)stream);
 }
 
 int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,

@@ -114,6 +114,31 @@ __device__ inline uint4 dequant8_w8(uint32_t w0, uint32_t w1, float s, float b) 
   return r;
 }
 
+// Code i of a little-endian bit stream of BITS-bit codes held in words w[0..];
+// i is a compile-time constant after unrolling, so this is one bit-field
+// extract, or one funnel shift and a mask where the code straddles two words.
+template <int BITS>
+__device__ inline uint32_t stream_code(const uint32_t* w, int i) {
+  const int bit = i * BITS, word = bit / 32, sh = bit % 32;
+  uint32_t c = w[word] >> sh;
+  if (sh + BITS > 32) c |= w[word + 1] << (32 - sh);
+  return c & ((1u << BITS) - 1u);
+}
+
+// codes 8c .. 8c+7 of a 32-code unit (BITS words) of MLX's 3-, 5- and 6-bit packs
+template <typename T, int BITS>
+__device__ inline uint4 dequant8_stream(const uint32_t* w, int c, float s, float b) {
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = __builtin_fmaf((float)stream_code<BITS>(w, 8 * c + i), s, b);
+  uint4 r;
+  r.x = T::pack2(v[0], v[1]);
+  r.y = T::pack2(v[2], v[3]);
+  r.z = T::pack2(v[4], v[5]);
+  r.w = T::pack2(v[6], v[7]);
+  return r;
+}
+
 // Exact 16-bit float images of codes, two per register.
 template <typename T>
 struct CodeFloat;
@@ -306,11 +331,18 @@ int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
 // y[M, N] += t @ bs^T, rounded to y's type (dtype: the type of t, bs and a 16-bit y)
 int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream);
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
-// the 128 x 128-tile kernel for a few hundred activation rows (K % 64 == 0)
+// the 128-column-tile kernel for a few hundred activation rows, and for any M when K % 64 == 32
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                    void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
 size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
+// the same kernel for 3, 5 and 6 bits (any M above one row; K % 32 == 0)
+int launch_qmm_mid_stream(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                          const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
+// y[M, K] = x[M, N] @ dequantize(wq[N, K]): the weight not transposed (N % 8 == 0)
+int launch_qmm_n(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                 const void* biases, int64_t K, int gs, int bits, void* y, int y_dtype, hipStream_t stream);
 // y = sum of `splits` float32 planes of M x N (+ bias), rounded to y's type; dtype is the type of bias and 16-bit y
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
                          int y_dtype, hipStream_t stream);

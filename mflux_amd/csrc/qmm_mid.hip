@@ -24,6 +24,7 @@
 #include <utility>
 
 #include "common.h"
+#include "tile_epilogue.h"
 
 namespace mfq {
 namespace {
@@ -36,8 +37,6 @@ constexpr int tile_m(int waves_m) { return 64 * waves_m; }
 constexpr int threads_of(int waves_m) { return 2 * waves_m * kWave; }
 constexpr int tile_x_bytes(int waves_m) { return tile_m(waves_m) * TK * 2; }
 constexpr int lds_bytes(int waves_m) { return 2 * (tile_x_bytes(waves_m) + kTileW); }  // both tiles, double buffered
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // 64 LDS banks of 4 bytes: a 128-bit access is conflict free when 16
 // consecutive lanes cover one 256-byte window (two rows).
@@ -53,14 +52,16 @@ __device__ inline void for_each_index(F&& f) {
   for_each_index_impl(f, std::make_integer_sequence<int, kN>{});
 }
 
-template <typename T>
-__device__ inline float lo_f32(uint32_t pk) { return T::to_f32((uint16_t)pk); }
-template <typename T>
-__device__ inline float hi_f32(uint32_t pk) { return T::to_f32((uint16_t)(pk >> 16)); }
-
 // kFast: scales and biases are read as 8-byte pieces (four consecutive groups
 // of a weight row) once per period of 4*GS/64 k steps; otherwise as one 2-byte
-// value per step.
+// value per step, and K may then end in half a step (K % 64 == 32, group size
+// 32): what lies past K enters LDS as zeros on both sides.
+//
+// BITS 3, 5 and 6 (mflux's -q 3/5/6, src/mflux/cli/defaults/defaults.py:63): a
+// row's codes are one little-endian bit stream, 32 codes in BITS whole words.
+// 256 threads take one such unit each (feature t/2, half t%2 of the step) and
+// cut the codes out at compile-time positions; with 512 threads the upper half
+// only copies x.  For these widths the kernel serves every M above one row.
 template <typename T, int GS, int BITS, bool kFast, int kWavesM>
 __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
@@ -73,7 +74,9 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   constexpr int kThreads = threads_of(kWavesM);
   constexpr int kTileX = tile_x_bytes(kWavesM);
   constexpr int kBuf = kTileX + kTileW;       // one buffer: the x tile, then the weight tile
-  constexpr int kCodes = TN * TK / kThreads;  // weights a thread dequantises per step: 32 or 16
+  constexpr bool kStream = BITS != 4 && BITS != 8;           // codes cut out of a bit stream
+  constexpr int kDeqThreads = kStream ? 256 : kThreads;      // threads that dequantise
+  constexpr int kCodes = TN * TK / kDeqThreads;  // weights such a thread dequantises per step: 32 or 16
   constexpr int kParts = TK / kCodes;         // threads per feature
   constexpr int kChunks = kCodes / 8;         // 8-code (16-byte) pieces it writes
   constexpr int kWords = kCodes * BITS / 32;  // 32-bit words of codes it loads
@@ -107,10 +110,13 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i)
     xoff[i] = ((uint32_t)min(m0 + (t >> 3) + kXPass * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
-  const int f = t / kParts, part = t % kParts;  // this thread's feature of the tile and part of the k step
+  const bool deq = t < kDeqThreads;             // uniform per wavefront
+  const int td = t % kDeqThreads;               // the other threads request what thread td does and drop it
+  const int f = td / kParts, part = td % kParts;  // this thread's feature of the tile and part of the k step
   const int hh = part * kCodes / 32;            // which half of the step (the group, for groups of 32)
   const uint32_t wrow = (uint32_t)min(n0 + f, N - 1);
-  const uint32_t woff = wrow * (uint32_t)(K * BITS / 8) + (uint32_t)(part * kCodes * BITS / 8);
+  constexpr int kPieceBytes = kCodes * BITS / 8;  // this thread's codes of one step
+  const uint32_t woff = wrow * (uint32_t)(K * BITS / 8) + (uint32_t)(part * kPieceBytes);
   const uint32_t soff = wrow * (uint32_t)(K / GS) * 2u;
   const char* xbytes = reinterpret_cast<const char*>(x);
   const char* wbytes = reinterpret_cast<const char*>(wq);
@@ -152,12 +158,20 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
         per[kSel].b = *reinterpret_cast<const uint2*>(bbytes + soff + (size_t)g0 * 2);
       }
     } else {
-      const int g0 = k0 / GS + (GS == 32 ? hh : 0);
+      const int g0 = min(k0 / GS + (GS == 32 ? hh : 0), K / GS - 1);
       g.s = *reinterpret_cast<const uint16_t*>(sbytes + soff + (size_t)g0 * 2);
       g.b = *reinterpret_cast<const uint16_t*>(bbytes + soff + (size_t)g0 * 2);
     }
-    const char* wsrc = wbytes + (size_t)k0 * BITS / 8 + woff;
-    if constexpr (kWords == 2) {
+    // a part past K (!kFast, K % 64 == 32) re-reads the row's last piece and is published as zeros
+    int wcol = k0 * BITS / 8;
+    if constexpr (!kFast) {
+      wcol = min(wcol, K * BITS / 8 - (part + 1) * kPieceBytes);
+    }
+    const char* wsrc = wbytes + woff + wcol;
+    if constexpr (kStream) {
+#pragma unroll
+      for (int l = 0; l < kWords; ++l) g.w[l] = *reinterpret_cast<const uint32_t*>(wsrc + 4 * l);
+    } else if constexpr (kWords == 2) {
       const uint2 v = *reinterpret_cast<const uint2*>(wsrc);
       g.w[0] = v.x;
       g.w[1] = v.y;
@@ -172,7 +186,11 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   };
   auto load_x_piece = [&](Stage& g, int q, int i) __attribute__((always_inline)) {
     const int k0 = kb + min(q, steps - 1) * TK;
-    g.x[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)k0 * 2 + xoff[i]);
+    int xcol = k0 * 2;
+    if constexpr (!kFast) {  // a piece past K re-reads the row's last one and is published as zeros
+      xcol = min(xcol, K * 2 - 16 * ((t & 7) + 1));
+    }
+    g.x[i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i] + xcol);
   };
   auto load = [&](auto sel, Stage& g, int q) __attribute__((always_inline)) {
     load_rest(sel, g, q);
@@ -202,18 +220,29 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   // Quarter c of publishing a step's registers to buffer `buf`: one 128-bit
   // piece of x and (in every quarter, or every other one) eight dequantised
   // weights.
-  auto publish_part = [&](const Stage& g, int c, float sc, float bi, int buf) __attribute__((always_inline)) {
+  // q: the step being published (its half past K, if any, becomes zeros).
+  auto publish_part = [&](const Stage& g, int q, int c, float sc, float bi, int buf) __attribute__((always_inline)) {
     char* xd = lds + buf * kBuf;
     char* wd = xd + kTileX;
-    *reinterpret_cast<u32x4*>(xd + wr_x + kXPass * TK * 2 * c) = g.x[c];
+    const int k0 = kb + q * TK;
+    u32x4 xv = g.x[c];
+    if constexpr (!kFast) {
+      if (k0 + 8 * (t & 7) >= K) xv = u32x4{0u, 0u, 0u, 0u};
+    }
+    *reinterpret_cast<u32x4*>(xd + wr_x + kXPass * TK * 2 * c) = xv;
     constexpr int kEvery = 4 / kChunks;
-    if (c % kEvery == 0) {
+    if (c % kEvery == 0 && deq) {
       const int cw = c / kEvery;
       uint4 v;
-      if constexpr (BITS == 4) {
+      if constexpr (kStream) {
+        v = dequant8_stream<T, BITS>(g.w, cw, sc, bi);
+      } else if constexpr (BITS == 4) {
         v = dequant8_w4<T>(g.w[cw], sc, bi);
       } else {
         v = dequant8_w8<T>(g.w[2 * cw], g.w[2 * cw + 1], sc, bi);
+      }
+      if constexpr (!kFast) {
+        if (k0 + part * kCodes >= K) v = make_uint4(0u, 0u, 0u, 0u);
       }
       *reinterpret_cast<uint4*>(wd + wr_w[cw]) = v;
     }
@@ -257,7 +286,7 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(af[sub & 1][j], bf[sub & 1][i], acc[i][j]);
-      publish_part(next, sub, sc, bi, buf ^ 1);
+      publish_part(next, p + 1, sub, sc, bi, buf ^ 1);
       // the registers just published are refilled for step p+3 right away
       load_x_piece(st[buf ^ 1], p + 3, sub);
       if (sub == 3) load_rest(sel_of(std::integral_constant<int, kE + 3>{}), st[buf ^ 1], p + 3);
@@ -274,7 +303,7 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     float sc, bi;
     scale_of(e0, st[0], sc, bi);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) publish_part(st[0], c, sc, bi, 0);
+    for (int c = 0; c < 4; ++c) publish_part(st[0], 0, c, sc, bi, 0);
     load(sel_of(std::integral_constant<int, 2>{}), st[0], 2);
     __syncthreads();
   }
@@ -317,105 +346,8 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     }
   }
 
-  // ---- epilogue: accumulator [i][j], register e holds output row
-  // m0 + 64wm + 32i + r and column n0 + 64wn + 32j + 8(e/4) + 4h + e%4.
-  // Every LDS tile is free now (the loop ended with a barrier); each wavefront
-  // transposes its block through a private region so that a global store
-  // instruction writes whole row segments.
-  const int mw = m0 + 64 * wm, nw = n0 + 64 * wn;
-  if (!y_is_f32 && (N & 7) == 0) {
-    constexpr int kStride = 144;  // 64 16-bit columns + 16 bytes of padding
-    char* stage = lds + wave * (64 * kStride);
-    uint16_t* yout = reinterpret_cast<uint16_t*>(y_item);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-      for (int eb = 0; eb < 4; ++eb) {
-        const int cl = 32 * j + 8 * eb + 4 * h;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (bias) {
-#pragma unroll
-          for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(nw + cl + c, N - 1)]);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          uint32_t pk[2];
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            pk[c] = T::pack2(acc[i][j][4 * eb + 2 * c], acc[i][j][4 * eb + 2 * c + 1]);
-            if (bias)  // second rounding, as a separate add on the 16-bit result would do
-              pk[c] = T::pack2(lo_f32<T>(pk[c]) + bv[2 * c], hi_f32<T>(pk[c]) + bv[2 * c + 1]);
-          }
-          *reinterpret_cast<uint2*>(stage + (32 * i + r) * kStride + cl * 2) = make_uint2(pk[0], pk[1]);
-        }
-      }
-    }
-    const int cg = nw + 8 * (lane & 7);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int rl = 8 * k + (lane >> 3);
-      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 16 * (lane & 7));
-      const int row = mw + rl;
-      if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
-    }
-  } else if (y_is_f32 && (N & 3) == 0) {
-    constexpr int kStride = 64 * 4 + 16;
-    char* stage = lds + wave * (32 * kStride);
-    float* yout = reinterpret_cast<float*>(y_item);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int eb = 0; eb < 4; ++eb) {
-          const int cl = 32 * j + 8 * eb + 4 * h;
-          float bv[4] = {0.f, 0.f, 0.f, 0.f};
-          if (bias) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[min(nw + cl + c, N - 1)]);
-          }
-          *reinterpret_cast<float4*>(stage + r * kStride + cl * 4) =
-              make_float4(acc[i][j][4 * eb] + bv[0], acc[i][j][4 * eb + 1] + bv[1], acc[i][j][4 * eb + 2] + bv[2],
-                          acc[i][j][4 * eb + 3] + bv[3]);
-        }
-      }
-      const int cg = nw + 4 * (lane & 15);
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int rl = 4 * k + (lane >> 4);
-        const float4 v = *reinterpret_cast<const float4*>(stage + rl * kStride + 16 * (lane & 15));
-        const int row = mw + 32 * i + rl;
-        if (row < M && cg < N) *reinterpret_cast<float4*>(yout + (int64_t)row * N + cg) = v;
-      }
-    }
-  } else {
-    // any N: element-wise guarded stores straight from the accumulators
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-      for (int eb = 0; eb < 4; ++eb) {
-        const int col = nw + 32 * j + 8 * eb + 4 * h;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int row = mw + 32 * i + r;
-          if (row >= M) continue;
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            if (col + c >= N) continue;
-            const float bv = bias ? T::to_f32(bias[col + c]) : 0.f;
-            const int64_t o = (int64_t)row * N + col + c;
-            if (y_is_f32) {
-              reinterpret_cast<float*>(y_item)[o] = acc[i][j][4 * eb + c] + bv;
-            } else {
-              uint16_t hv = T::from_f32(acc[i][j][4 * eb + c]);
-              if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
-              reinterpret_cast<uint16_t*>(y_item)[o] = hv;
-            }
-          }
-        }
-      }
-    }
-  }
+  // ---- epilogue: every LDS tile is free now (the loop ended with a barrier)
+  store_block_64x64<T>(acc, lds, wave, lane, m0 + 64 * wm, n0 + 64 * wn, M, N, bias, y_item, y_is_f32);
 }
 
 struct MidPlan {
@@ -434,13 +366,13 @@ inline int waves_m_of(int64_t M) { return M <= 128 ? 2 : 4; }
 // while the work items are fewer than the compute units and the cut keeps them
 // within what runs at once.
 inline MidPlan plan_mid(int64_t M, int64_t N, int64_t K, int period, int cus) {
-  const int steps = (int)(K / TK);
+  const int steps = (int)((K + TK - 1) / TK);  // K % 64 == 32: the last step is half empty
   const int waves_m = waves_m_of(M);
   const int tm = tile_m(waves_m);
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + TN - 1) / TN);
   const int64_t slots = waves_m == 2 ? 2 * (int64_t)cus : cus;
   MidPlan plan{1, steps};
-  if (steps % period != 0) return plan;
+  if (K % TK || steps % period != 0) return plan;
   for (int s = 2; s <= steps / 8 && tiles * plan.splits < cus && tiles * s <= slots; ++s)
     if (steps % s == 0 && (steps / s) % period == 0) plan = MidPlan{s, steps / s};
   return plan;
@@ -475,10 +407,10 @@ template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
                hipStream_t stream, LowRank lr) {
-  const int64_t steps = K / TK;
+  const int64_t steps = (K + TK - 1) / TK;
   constexpr int kPer = 4 * GS / TK;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
-  if (!(steps % kPer == 0 && aligned8))
+  if (!(K % TK == 0 && steps % kPer == 0 && aligned8))
     return launch_tile<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
                                            stream, lr);
   const MidPlan plan = plan_mid(M, N, K, kPer, compute_units());
@@ -492,13 +424,24 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
 }
 
+// This file is compiled twice: as it is for 4 and 8 bits, and through
+// qmm_mid_stream.hip (which defines MFQ_MID_STREAM and includes it) for the 3-,
+// 5- and 6-bit packs, so that the two sets of instantiations build in parallel.
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                 const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
                 hipStream_t stream, LowRank lr) {
+#ifdef MFQ_MID_STREAM
+  if (bits == 3)
+    return launch_one<T, GS, 3>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+  if (bits == 5)
+    return launch_one<T, GS, 5>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+  return launch_one<T, GS, 6>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+#else
   if (bits == 4)
     return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
   return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+#endif
 }
 
 template <typename T>
@@ -517,8 +460,12 @@ int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const voi
 
 }  // namespace
 
+#ifdef MFQ_MID_STREAM
+int launch_qmm_mid_stream(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                          const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+#else
 size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
-  if (K % TK) return 0;
   const MidPlan plan = plan_mid(M, N, K, period_of(gs), compute_units());
   return plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
 }
@@ -526,6 +473,10 @@ size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                    void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+  if (bits != 4 && bits != 8)
+    return launch_qmm_mid_stream(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
+                                 workspace_bytes, stream, low_rank);
+#endif
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if (dtype == MFQ_BF16)

@@ -348,6 +348,18 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
   }
 }
 
+// code * scale + bias as mx.dequantize evaluates it: an element-wise multiply and
+// an element-wise add on arrays of the output type, so the product is rounded
+// to that type before the bias is added and the sum is rounded again by the
+// store (float32 output: the two float32 operations, never fused).  The matmul
+// kernels do not go through this; they round fma(code, scale, bias) once.
+template <typename TO>
+__device__ inline float dequant_value(float q, float s, float b) {
+  float p = q * s;
+  if constexpr (sizeof(typename TO::storage) == 2) p = TO::to_f32(TO::from_f32(p));
+  return p + b;
+}
+
 template <typename TS, typename TO, int GS, int BITS>
 __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restrict__ wq,
                                                          const typename TS::storage* __restrict__ scales,
@@ -374,7 +386,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const uint32_t* __restr
     }
     float r[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_fmaf(q[i], s, b);
+    for (int i = 0; i < 8; ++i) r[i] = dequant_value<TO>(q[i], s, b);
     if constexpr (sizeof(typename TO::storage) == 2) {
       uint4 o;
       o.x = TO::pack2(r[0], r[1]);
@@ -426,7 +438,7 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(const uint32_t* __
     }
     float r[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_fmaf(q[i], s, b);
+    for (int i = 0; i < 8; ++i) r[i] = dequant_value<TO>(q[i], s, b);
     const int64_t cd = dst0 + c;
     if constexpr (sizeof(typename TO::storage) == 2) {
       uint4 o;
@@ -476,7 +488,7 @@ __global__ __launch_bounds__(256) void dequantize_stream_kernel(const uint32_t* 
       const int bit = e * BITS, word = bit / 32, sh = bit % 32;
       uint32_t code = w[word] >> sh;
       if (sh + BITS > 32) code |= w[word + 1] << (32 - sh);
-      r[e] = __builtin_fmaf((float)(code & ((1u << BITS) - 1u)), s, b);
+      r[e] = dequant_value<TO>((float)(code & ((1u << BITS) - 1u)), s, b);
     }
     if constexpr (sizeof(typename TO::storage) == 2) {
 #pragma unroll

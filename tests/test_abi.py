@@ -93,8 +93,22 @@ def test_argument_validation_needs_no_device():
     assert call(wq=None) == E["null"]
     assert call(x=base + 4) == E["align"]
     assert call(gs=16) == E["group"]
-    assert call(bits=5) == -8                        # 3, 5, 6 bits: a fused kernel for one activation row only
-    assert call(bits=5, M=1, K=100) == E["shape"]    # ... which validates its arguments like the others
+    assert call(bits=5, y=base + 2) == E["align"]    # 3, 5, 6 bits, several rows: the GEMM writes y in 16-byte pieces
+    assert call(bits=5, M=1, K=100) == E["shape"]    # the odd widths validate their arguments like the others
+    n = lib.mfq_qmm_n                                 # the untransposed product: x [M, N], y [M, K]
+
+    def call_n(x=base, xd=_lib.BF16, M=4, N=8, wq=base, s=base, b=base, sd=_lib.BF16, K=128, gs=64, bits=4, y=base,
+               yd=_lib.BF16):
+        return n(x, xd, M, N, wq, s, b, sd, K, gs, bits, y, yd, None)
+
+    assert call_n(xd=_lib.F32) == E["dtype"]
+    assert call_n(yd=_lib.F16) == E["dtype"]
+    assert call_n(K=100) == E["shape"]
+    assert call_n(N=0) == E["shape"]
+    assert call_n(s=None) == E["null"]
+    assert call_n(y=base + 8) == E["align"]
+    assert call_n(bits=7) == E["bits"]
+    assert call_n(N=12) == E["unsupported"]          # x rows are read in 16-byte pieces
 
     # the LoRA entry points: the rank comes in steps of 16 with both matrices present and aligned
     lr = lib.mfq_qmm_t_low_rank
@@ -150,3 +164,22 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmfq.so"))
     with pytest.raises(ImportError, match="no CPU or PyTorch fallback"):
         _lib.load()
+
+
+def test_torch_ops_are_registered_and_refuse_cpu_tensors():
+    """csrc/torch_ops.cpp: every op mflux_amd.core calls exists under
+    torch.ops.mfq, only for the HIP backend (a CPU tensor is refused by the
+    dispatcher: there is nothing to fall back to)."""
+    import torch
+
+    from mflux_amd import _lib
+
+    ops = _lib.ops()
+    for name in ("quantize_affine", "dequantize_affine", "dequantize_rows", "qmm_t", "qmv_silu", "low_rank_add_"):
+        assert hasattr(ops, name), name
+    with pytest.raises(NotImplementedError, match="CPU"):
+        ops.quantize_affine(torch.zeros(2, 64, dtype=torch.bfloat16), 64, 4)
+    with pytest.raises(NotImplementedError, match="CPU"):
+        ops.qmm_t(torch.zeros(2, 64, dtype=torch.bfloat16), torch.zeros(4, 8, dtype=torch.int32).view(torch.uint32),
+                  torch.zeros(4, 1, dtype=torch.bfloat16), torch.zeros(4, 1, dtype=torch.bfloat16), None, 64, 4,
+                  torch.bfloat16, None, None)

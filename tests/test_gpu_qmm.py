@@ -401,8 +401,9 @@ def test_qmm_k_not_multiple_of_64(oracle, bits):
 @pytest.mark.parametrize("bits", [3, 5, 6])
 @pytest.mark.parametrize("M", [1, 300])
 def test_odd_bit_widths_matmul(oracle, bits, M):
-    """3, 5, 6 bits: dequantize kernel + library GEMM, to the same tolerance,
-    through the functional API and through a QuantizedLinear."""
+    """3, 5, 6 bits, one row (its own kernel) and a few hundred (the
+    128-column-tile GEMM on the bit stream), through the functional API and
+    through a QuantizedLinear."""
     import mflux_amd
     from gpu_util import to_dev
     from mflux_amd import nn as qnn
@@ -427,7 +428,7 @@ def test_odd_bit_widths_matmul(oracle, bits, M):
 def test_odd_bit_widths_single_row_kernel(oracle, bits, gs, K):
     """3, 5, 6 bits with one activation row: the fused kernel (one to four units
     of 32 codes per lane, whole and partial last rounds, all group sizes) and,
-    for K = 8256, the first shape beyond it (dequantize + library GEMM)."""
+    for K = 8256, the first shape beyond it (the GEMM kernel with one row)."""
     import mflux_amd
     from gpu_util import to_dev, u32_to_dev
 
@@ -466,22 +467,24 @@ def test_odd_bit_widths_one_hot(oracle, bits):
 
 
 def test_odd_bit_widths_c_abi_coverage(oracle):
-    """mfq_qmm_t takes 3-, 5- and 6-bit weights for one activation row with rows
-    of at most 8192 codes, and says MFQ_EUNSUPPORTED for anything else."""
+    """mfq_qmm_t takes 3-, 5- and 6-bit weights for any number of rows: one row of
+    at most 8192 codes on its own kernel, the rest on the GEMM kernel."""
     from gpu_util import to_dev, u32_to_dev
     from mflux_amd import _lib
 
     o = oracle
     lib = _lib.load()
     for bits in (3, 5, 6):
-        for M, K, expect in ((1, 3072, 0), (2, 3072, _lib.MFQ_EUNSUPPORTED), (1, 8256, _lib.MFQ_EUNSUPPORTED)):
-            x, wq, s, b, _ = _case(o, 53, M, K, 16, bits, gs=32, with_bias=False)
+        for M, K in ((1, 3072), (2, 3072), (1, 8256)):
+            args = _case(o, 53, M, K, 16, bits, gs=32, with_bias=False)
+            x, wq, s, b, _ = args
             xd, wd, sd, bd = to_dev(x, o.BF16), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16)
             y = torch.empty((M, 16), dtype=torch.bfloat16, device="cuda")
             rc = lib.mfq_qmm_t(xd.data_ptr(), _lib.BF16, M, K, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), _lib.BF16,
                                None, 16, 32, bits, y.data_ptr(), _lib.BF16, None)
             torch.cuda.synchronize()
-            assert rc == expect, (bits, M, K, rc)
+            assert rc == 0, (bits, M, K, rc)
+            _assert_close(y, _ref(o, *args, bits, 32))
 
 
 def test_odd_bit_widths_single_row_f16(oracle):
@@ -794,3 +797,41 @@ def test_shape_sweep_against_oracle(oracle, case):
     # average, |x row|_2 times the weights' standard deviation.
     x_norm = np.linalg.norm(o.bf16_bits_to_f32(args[0]).astype(np.float64), axis=-1, keepdims=True)
     _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs), row_floor=0.02 * x_norm)
+
+
+def test_torch_ops_and_ctypes_routes_agree_bit_for_bit(oracle):
+    """The two ways into libmfq -- torch.ops.mfq (what mflux_amd.core uses) and the
+    C ABI through ctypes -- run the same kernels on the same stream: quantize,
+    dequantize and the product (matvec, medium-M with a K split, large-M) come
+    out bit-identical."""
+    from gpu_util import to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib, ops = _lib.load(), _lib.ops()
+    stream = torch.cuda.current_stream().cuda_stream
+    for M, K, N, bits in ((1, 3072, 512, 8), (300, 2048, 1024, 4), (700, 512, 1536, 8)):
+        x = to_dev(o.f32_to_bf16_bits(seeded(81, 0, (M, K), 1.0)), o.BF16)
+        w = to_dev(o.f32_to_bf16_bits(seeded(81, 1, (N, K), 0.02)), o.BF16)
+        bias = to_dev(o.f32_to_bf16_bits(seeded(81, 2, (N,), 0.02)), o.BF16)
+        wq, s, b = ops.quantize_affine(w, 64, bits)
+        wq_c = torch.empty_like(wq)
+        s_c, b_c = torch.empty_like(s), torch.empty_like(b)
+        assert lib.mfq_quantize_affine(w.data_ptr(), _lib.BF16, N, K, 64, bits, wq_c.data_ptr(), s_c.data_ptr(),
+                                       b_c.data_ptr(), stream) == 0
+        assert torch.equal(wq.view(torch.int32), wq_c.view(torch.int32))
+        assert torch.equal(s.view(torch.int16), s_c.view(torch.int16)) and torch.equal(b.view(torch.int16), b_c.view(torch.int16))
+        d = ops.dequantize_affine(wq, s, b, 64, bits, torch.bfloat16)
+        d_c = torch.empty_like(d)
+        assert lib.mfq_dequantize_affine(wq.data_ptr(), s.data_ptr(), b.data_ptr(), _lib.BF16, N, K, 64, bits,
+                                         d_c.data_ptr(), _lib.BF16, stream) == 0
+        assert torch.equal(d.view(torch.int16), d_c.view(torch.int16))
+        y, ok = ops.qmm_t(x, wq, s, b, bias, 64, bits, torch.bfloat16, None, None)
+        assert ok
+        need = lib.mfq_qmm_t_workspace_bytes(M, K, N, 64, bits)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        y_c = torch.empty_like(y)
+        assert lib.mfq_qmm_t_ws(x.data_ptr(), _lib.BF16, M, K, wq.data_ptr(), s.data_ptr(), b.data_ptr(), _lib.BF16,
+                                bias.data_ptr(), N, 64, bits, y_c.data_ptr(), _lib.BF16, ws.data_ptr(), need, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), y_c.view(torch.int16)), (M, K, N, bits)
