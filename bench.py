@@ -35,14 +35,17 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# L2 <-> fabric bytes per GEMM launch (read + written), mean over the two
-# shapes of the step, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# plain copy of known size; the figures and the commands are in
-# profiles/qmm_w4a16_flux_single_block_m4608.md.  Not measurable from inside
-# this script.
-TRAFFIC_BYTES_PER_LAUNCH = ((561.9e6 + 208.8e6) + (503.6e6 + 33.0e6)) / 2
+# L2 <-> fabric bytes per launch are hardware counters (rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by a plain copy of known size) and cannot be read from inside
+# this script: `roofline.traffic` is taken from the line `traffic_bytes_per_launch:
+# <number>` of the committed summary of that profile, and says so.
+TRAFFIC_PROFILES = {
+    "gemm": "profiles/qmm_w4a16_flux_single_block_m4608.md",
+    "gemv": "profiles/qmv_w8_adaln_3072x18432.md",
+}
 
 M_TOKENS = 4608
+CONFIG = 3  # the benchmark configuration of the step: seeds are 1000 * config + tensor index
 LINEARS = (("linear1", 3072, 21504), ("linear2", 15360, 3072))  # (name, K, N)
 GS, BITS = 64, 4
 
@@ -53,6 +56,103 @@ def qmm_bytes(M, K, N, bits, bias=False):
 
 def quantize_bytes(N, K, bits):
     return 2 * N * K + N * K * bits // 8 + 4 * N * K // 64
+
+
+def profiled_traffic(which):
+    """(bytes per launch, source) from the committed counter profile, or (None, reason)."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILES[which])
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0]), (
+                        f"{TRAFFIC_PROFILES[which]} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE of an earlier run of "
+                        "this command, scaled by a 256 MiB copy; not counted in this run)")
+    except OSError:
+        pass
+    return None, f"{TRAFFIC_PROFILES[which]} holds no traffic_bytes_per_launch line"
+
+
+def seeded_bf16(torch, dev, config, index, shape, std):
+    """The benchmark's input convention: numpy default_rng(1000 * config + index),
+    float32 normals scaled by std, rounded once to bfloat16."""
+    import numpy as np
+
+    rng = np.random.default_rng(1000 * config + index)
+    a = rng.standard_normal(shape, dtype=np.float32)
+    if std != 1.0:
+        a *= np.float32(std)
+    return torch.from_numpy(a).to(dev).to(torch.bfloat16)
+
+
+class Telemetry:
+    """Socket power and shader clock of GPU 0 sampled from sysfs by a thread
+    while a timed region runs (ordinary user, nothing is changed)."""
+
+    def __init__(self, period=0.01):
+        import glob
+
+        self.period = period
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.power = next((os.path.join(d, f) for d in hw for f in ("power1_average", "power1_input")
+                           if os.path.exists(os.path.join(d, f))), None)
+        self.cap = next((os.path.join(d, "power1_cap") for d in hw if os.path.exists(os.path.join(d, "power1_cap"))),
+                        None)
+        sclk = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.sclk = sclk[0] if sclk else None
+        self.samples = []
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return None
+
+    def _sample(self):
+        watts = mhz = None
+        txt = self._read(self.power) if self.power else None
+        if txt:
+            watts = int(txt) / 1e6
+        txt = self._read(self.sclk) if self.sclk else None
+        for line in (txt or "").splitlines():
+            if line.rstrip().endswith("*"):
+                digits = "".join(ch for ch in line.split(":", 1)[1] if ch.isdigit())
+                mhz = int(digits) if digits else None
+        return watts, mhz
+
+    def __enter__(self):
+        import threading
+
+        self._stop = threading.Event()
+
+        def run():
+            while not self._stop.is_set():
+                self.samples.append(self._sample())
+                self._stop.wait(self.period)
+
+        self._thread = threading.Thread(target=run, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def summary(self):
+        watts = [w for w, _ in self.samples if w is not None]
+        mhz = [m for _, m in self.samples if m is not None]
+        cap = self._read(self.cap) if self.cap else None
+        return {
+            "samples": len(self.samples),
+            "socket_power_w_mean": round(sum(watts) / len(watts), 1) if watts else None,
+            "socket_power_w_max": round(max(watts), 1) if watts else None,
+            "power_cap_w": int(cap) / 1e6 if cap else None,
+            "sclk_mhz_mean": round(sum(mhz) / len(mhz), 1) if mhz else None,
+            "sclk_mhz_min": min(mhz) if mhz else None,
+            "source": "sysfs hwmon power1 and pp_dpm_sclk of card 0, sampled every 10 ms over the timed region",
+        }
 
 
 def event_ms(fn, iters, torch):
@@ -155,7 +255,7 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    gen = torch.Generator(device=dev).manual_seed(3000)
+    gen = torch.Generator(device=dev).manual_seed(3000)  # for the side legs only; the step's operands are seeded by numpy
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(7)
@@ -167,9 +267,9 @@ def main():
     # ---- operands of the step, resident in HBM --------------------------------
     ops = []
     quant_ms = {}
-    for name, K, N in LINEARS:
-        x = torch.randn(M_TOKENS, K, device=dev, generator=gen).to(torch.bfloat16)
-        w = (torch.randn(N, K, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    for lin, (name, K, N) in enumerate(LINEARS):
+        x = seeded_bf16(torch, dev, CONFIG, 10 * lin + 0, (M_TOKENS, K), 1.0)
+        w = seeded_bf16(torch, dev, CONFIG, 10 * lin + 1, (N, K), 0.02)
         wq, s, b = mflux_amd.quantize(w, GS, BITS)
         copies = [w] + [w.clone() for _ in range(3)]  # > 256 MB in rotation: cold reads
         turn = {"i": 0}
@@ -190,15 +290,27 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(args.steps):
-        step()
-    stop.record()
+    # The chip needs some hundred launches under load before clocks and power settle (the first
+    # batches run up to a tenth slower), so beyond the requested warm-up steps, batches of untimed
+    # steps run until two in a row agree within 1 % (at most 40 batches of 10).
+    settle, prev = [], None
+    for _ in range(40):
+        ms = event_ms(step, 10, torch)
+        settle.append(round(ms, 4))
+        if prev is not None and abs(ms - prev) <= 0.01 * prev:
+            break
+        prev = ms
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    with Telemetry() as telemetry:
+        t0 = time.perf_counter()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(args.steps):
+            step()
+        stop.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms_per_step = start.elapsed_time(stop) / args.steps
 
@@ -206,6 +318,7 @@ def main():
     value = flops / (ms_per_step * 1e-3) / 1e12
     launches = len(LINEARS)
     achieved = flops / (kernel_ms_per_step * 1e-3) / 1e12  # = mean flops per launch / mean launch duration
+    traffic, traffic_source = profiled_traffic("gemm")
     roofline = {
         "kernel": "qmm_kernel<BF16,64,4>",
         "bound": "mfma",
@@ -213,9 +326,12 @@ def main():
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+        "traffic": traffic,
+        "traffic_source": traffic_source,
         "avg_launch_us": round(kernel_ms_per_step * 1e3 / launches, 2),
         "flops_per_launch": flops / launches,
+        "telemetry": telemetry.summary(),
+        "settling_ms_per_step": settle,
     }
 
     # per-shape GEMM timings
@@ -272,18 +388,19 @@ def main():
     # ---- secondary: GEMV of the adaLN modulation shape, cold weights -----------
     gemv = {}
     Kg, Ng = 3072, 18432
+    # configuration 2: W ~ N(0, 0.02) [18432, 3072], eight different matrices (seeds 2001..2008) so that the
+    # weights in rotation exceed the 256 MB memory-side cache; at 4 bits the eight are stored twice
+    gemv_w16 = [] if args.no_secondary else [seeded_bf16(torch, dev, 2, 1 + i, (Ng, Kg), 0.02) for i in range(8)]
     for bits_g in (() if args.no_secondary else (8, 4)):
-        n_buf = 8 if bits_g == 8 else 16  # more than 256 MB in rotation
-        bufs = []
-        for i in range(n_buf):
-            w = (torch.randn(Ng, Kg, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
-            bufs.append(mflux_amd.quantize(w, GS, bits_g))
-            del w
-        bias = (torch.randn(Ng, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+        bufs = [mflux_amd.quantize(w, GS, bits_g) for w in gemv_w16]
+        if bits_g == 4:
+            bufs += [tuple(t.clone() for t in buf) for buf in bufs]
+        n_buf = len(bufs)  # more than 256 MB in rotation
+        bias = seeded_bf16(torch, dev, 2, 100, (Ng,), 0.02)
         res = {}
         for Mg in (1, 4):
-            temb = torch.randn(Mg, Kg, device=dev, generator=gen)
-            xg = torch.nn.functional.silu(temb).to(torch.bfloat16)
+            temb = seeded_bf16(torch, dev, 2, 0, (Mg, Kg), 1.0)
+            xg = mflux_amd.silu(temb)  # x = SiLU(temb), evaluated as MLX's nn.silu does on bfloat16
             state = {"i": 0}
 
             def gemv_call():
@@ -299,7 +416,7 @@ def main():
                              "weights": f"rotating over {n_buf} buffers ({n_buf * Ng * Kg * bits_g // 8 >> 20} MiB)"}
         # the whole modulation call linear(silu(temb)) at M = 1: the activation inside the matvec
         # kernel against an elementwise pass in front of it (what the reference runs)
-        temb16 = torch.randn(1, Kg, device=dev, generator=gen).to(torch.bfloat16)
+        temb16 = seeded_bf16(torch, dev, 2, 0, (1, Kg), 1.0)
         state = {"i": 0}
 
         def fused_call():
@@ -330,11 +447,12 @@ def main():
         del picks, wq_all, s_all, b_all, bias_all
         res["M1_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
                                "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
-        temb16 = torch.randn(4, Kg, device=dev, generator=gen).to(torch.bfloat16)  # the same for a batch of four
+        temb16 = seeded_bf16(torch, dev, 2, 0, (4, Kg), 1.0)  # the same for a batch of four
         res["M4_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
                                "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
         gemv[f"w{bits_g}"] = res
         del bufs
+    del gemv_w16
 
     # ---- secondary: the text stream of a joint block (M = 512) -----------------
     medium = {}
@@ -359,8 +477,10 @@ def main():
     gemv_roofline = None
     if "w8" in gemv:
         m1 = gemv["w8"]["M1"]
+        gemv_traffic, gemv_traffic_source = profiled_traffic("gemv")
         gemv_roofline = {"kernel": "qmv_dot_kernel<BF16,8,3>", "bound": "hbm", "achieved": m1["GB/s"],
-                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": m1["frac_hbm"], "traffic": 62.7e6 + 0.04e6,
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": m1["frac_hbm"], "traffic": gemv_traffic,
+                         "traffic_source": gemv_traffic_source,
                          "avg_launch_us": m1["us"], "bytes_per_launch": m1["bytes"]}
     out = {
         "metric": "W4A16 qmatmul TFLOP/s @ FLUX single-block M=4608",

@@ -57,6 +57,44 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def sanitize_abi(verbose: bool = False) -> str:
+    """Host-sanitizer run of the C ABI's argument validation: abi.hip compiled
+    with AddressSanitizer and UndefinedBehaviorSanitizer on its host side (the
+    device side is untouched), linked with the ordinary kernel objects and the
+    driver csrc/abi_sanitize_check.cpp, and run.  Every call in the driver is
+    refused before a launch, so no GPU is needed.  Needs the objects of
+    build_library().  Returns the driver's output; raises if it reports a
+    finding."""
+    san = os.path.join(CSRC, "_san")
+    os.makedirs(san, exist_ok=True)
+    host_san = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+                "-Xarch_host", "-fno-sanitize-recover=all", "-Xarch_host", "-fno-omit-frame-pointer", "-g"]
+    abi_o = os.path.join(san, "abi.o")
+    drv_o = os.path.join(san, "abi_sanitize_check.o")
+    exe = os.path.join(san, "abi_sanitize_check")
+    others = [os.path.join(CSRC, os.path.splitext(s)[0] + ".o") for s in SOURCES if s != "abi.hip"]
+    missing = [o for o in others if not os.path.exists(o)]
+    if missing:
+        raise RuntimeError(f"run build_library() first: {missing[0]} is missing")
+    steps = [
+        [hipcc(), *HIPCC_FLAGS, *host_san, "-c", os.path.join(CSRC, "abi.hip"), "-o", abi_o],
+        [hipcc(), "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-c",
+         os.path.join(CSRC, "abi_sanitize_check.cpp"), "-o", drv_o],
+        [hipcc(), "--offload-arch=gfx950", "-fsanitize=address,undefined", "-o", exe, drv_o, abi_o, *others],
+    ]
+    for cmd in steps:
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"{' '.join(cmd[:3])} ... failed:\n{res.stdout}\n{res.stderr}")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0", UBSAN_OPTIONS="print_stacktrace=1")
+    res = subprocess.run([exe], capture_output=True, text=True, env=env)
+    if res.returncode != 0:
+        raise RuntimeError(f"abi_sanitize_check reported a finding (exit {res.returncode}):\n{res.stdout}\n{res.stderr}")
+    if verbose:
+        print(res.stdout.strip())
+    return res.stdout
+
+
 OPS_PATH = os.path.join(CSRC, "libmfq_torch.so")
 
 
@@ -82,5 +120,10 @@ def build_torch_ops(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    build_library(verbose=True)
-    build_torch_ops(verbose=True)
+    import sys
+
+    if "--sanitize-abi" in sys.argv:
+        sanitize_abi(verbose=True)
+    else:
+        build_library(verbose=True)
+        build_torch_ops(verbose=True)

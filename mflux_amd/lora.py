@@ -146,7 +146,10 @@ def _bake(base: torch.nn.Module, loras: list[LoRALinear], requantize: bool) -> N
         # all adapters at once, so that the weight is requantized a single time
         full = core.dequantize(base.weight, base.scales, base.biases, base.group_size, base.bits)
         baked = (full.float() + sum(deltas).to(full.device)).to(full.dtype)
-        base.weight, base.scales, base.biases = core.quantize(baked, base.group_size, base.bits, base.mode)
+        # written into the layer's own tensors: they may be views of a stack (nn.concat_quantized)
+        for old, new in zip((base.weight, base.scales, base.biases),
+                            core.quantize(baked, base.group_size, base.bits, base.mode)):
+            old.copy_(new)
         return
     with torch.no_grad():
         for delta in deltas:   # one rounded add per adapter, as the reference does

@@ -162,7 +162,11 @@ def concat_quantized(layers: list[QuantizedLinear], share_storage: bool = False)
     the result with ``split`` / slicing (views, no copy).  The inputs are left
     untouched (their tensors are copied) unless ``share_storage`` is set: then
     every input layer's tensors become views of the stacked ones, so the stack
-    costs no memory and the layers keep working on their own.
+    costs no memory and the layers keep working on their own.  The views stay
+    in step with the stack as long as new values are written INTO the layers'
+    tensors: ``weights.update_module`` and ``lora.bake_and_strip_lora`` copy in
+    place when shape and dtype are unchanged; assigning a fresh tensor to
+    ``layer.weight`` detaches that layer from the stack, so stack after loading.
 
     The same serves the adaLN modulation linears of a whole model
     (src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:12 in

@@ -100,11 +100,13 @@ def tree_unflatten(items: Iterable[tuple[str, Any]]) -> Any:
 
 def update_module(model: torch.nn.Module, tree: Any, strict: bool = False) -> set[str]:
     """Sets parameters and buffers of ``model`` from a nested tree (or a flat
-    ``{dotted path: tensor}`` dict), replacing the stored tensor rather than
-    copying into it, so dtype and shape follow the new value (a quantized
-    layer's ``weight`` is uint32 of a different shape than the float one).
-    Paths that name nothing in the model are skipped unless ``strict``.
-    Returns the set of paths that were set."""
+    ``{dotted path: tensor}`` dict).  A value of the stored tensor's shape and
+    dtype is copied into it, so that views of that storage stay valid (the
+    layers of ``nn.concat_quantized(..., share_storage=True)`` are views of the
+    stack); any other value replaces the stored tensor, so dtype and shape
+    follow it (a quantized layer's ``weight`` is uint32 of a different shape
+    than the float one).  Paths that name nothing in the model are skipped
+    unless ``strict``.  Returns the set of paths that were set."""
     done: set[str] = set()
     for path, value in tree_flatten(tree):
         if not isinstance(value, torch.Tensor):
@@ -118,14 +120,17 @@ def update_module(model: torch.nn.Module, tree: Any, strict: bool = False) -> se
             if strict:
                 raise ValueError(f"weight '{path}' does not match any parameter of the model")
             continue
-        if name in owner._parameters:
-            old = owner._parameters[name]
+        params = name in owner._parameters
+        old = owner._parameters[name] if params else owner._buffers[name]
+        if old is not None and old.shape == value.shape and old.dtype == value.dtype:
+            with torch.no_grad():
+                old.copy_(value)
+        elif params:
             if old is not None:
                 value = value.to(old.device)
             trainable = bool(old is not None and old.requires_grad and value.is_floating_point())
             owner._parameters[name] = torch.nn.Parameter(value, requires_grad=trainable)
         else:
-            old = owner._buffers[name]
             owner._buffers[name] = value.to(old.device) if old is not None else value
         done.add(path)
     return done
@@ -256,15 +261,19 @@ def library_version() -> str:
 
 
 def split_weights(weights: dict[str, torch.Tensor], max_bytes: int = MAX_SHARD_BYTES) -> list[dict]:
-    """Greedy, order-preserving shards: a tensor that would take the running
-    shard past ``max_bytes`` starts the next one (an over-sized tensor gets a
-    shard of its own; no empty shard is produced)."""
+    """Greedy, order-preserving shards, statement for statement
+    ``ModelSaver._split_weights``
+    (src/mflux/models/common/weights/saving/model_saver.py:86-99): a tensor that
+    would take the running shard past ``max_bytes`` closes it and starts the
+    next one.  As in the reference the running shard is closed even when it is
+    still empty, so a first tensor larger than ``max_bytes`` leaves an empty
+    shard 0 in front of its own; only a trailing empty shard is dropped."""
     shards: list[dict] = []
     shard: dict = {}
     size = 0
     for key, value in weights.items():
         nbytes = value.numel() * value.element_size()
-        if shard and size + nbytes > max_bytes:
+        if size + nbytes > max_bytes:
             shards.append(shard)
             shard, size = {}, 0
         shard[key] = value
@@ -297,11 +306,21 @@ def save_weights(base_path: str | Path, bits: int | None, model: torch.nn.Module
 
 def save_model(model: Any, bits: int | None, base_path: str | Path, weight_definition) -> None:
     """One directory per component, named by the component's ``hf_subdir``; the
-    component is the attribute ``model_attr`` (or ``name``) of ``model``."""
+    component is the attribute ``model_attr`` (or ``name``) of ``model``.  As
+    ``ModelSaver.save_model`` does
+    (src/mflux/models/common/weights/saving/model_saver.py:38-41), LoRA wrappers
+    are baked into their base layers and stripped first (in place: the model
+    keeps the baked layers), so that the saved keys are the base model's."""
+    from .lora import bake_and_strip_lora
+
     for c in weight_definition.get_components():
-        component = getattr(model, c.model_attr or c.name, None)
+        attr = c.model_attr or c.name
+        component = getattr(model, attr, None)
         if component is not None:
-            save_weights(base_path, bits, component, c.hf_subdir)
+            stripped = bake_and_strip_lora(component)
+            if stripped is not component:  # the component itself was a wrapper
+                setattr(model, attr, stripped)
+            save_weights(base_path, bits, stripped, c.hf_subdir)
 
 
 def try_load_saved_format(path: str | Path, device: str | torch.device = "cpu"):

@@ -183,3 +183,12 @@ def test_torch_ops_are_registered_and_refuse_cpu_tensors():
         ops.qmm_t(torch.zeros(2, 64, dtype=torch.bfloat16), torch.zeros(4, 8, dtype=torch.int32).view(torch.uint32),
                   torch.zeros(4, 1, dtype=torch.bfloat16), torch.zeros(4, 1, dtype=torch.bfloat16), None, 64, 4,
                   torch.bfloat16, None, None)
+
+
+def test_abi_validation_clean_under_host_sanitizers():
+    """The C ABI's argument validation (csrc/abi.hip, host side) under
+    AddressSanitizer and UndefinedBehaviorSanitizer: every refusal of
+    csrc/abi_sanitize_check.cpp comes back with its status and no finding."""
+    from mflux_amd import _build
+
+    assert "every refusal clean" in _build.sanitize_abi()

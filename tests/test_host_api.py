@@ -351,6 +351,11 @@ def test_split_weights_greedy_order():
     shards = W.split_weights(t, max_bytes=100)
     assert [list(s) for s in shards] == [["t0"], ["t1", "t2"], ["t3"], ["t4", "t5"]]
     assert W.split_weights({}, 100) == []
+    # a first tensor beyond the limit: the reference closes the still empty shard in front of it
+    # (model_saver.py:92-95 has no "if shard"), so its own shard is number 1; a last one is never empty
+    big = {"a": torch.zeros(150, dtype=torch.uint8), "b": torch.zeros(10, dtype=torch.uint8)}
+    assert [list(s) for s in W.split_weights(big, max_bytes=100)] == [[], ["a"], ["b"]]
+    assert [list(s) for s in W.split_weights({"a": torch.zeros(150, dtype=torch.uint8)}, max_bytes=100)] == [[], ["a"]]
 
 
 def test_foreign_directory_is_not_our_format(tmp_path):
@@ -404,3 +409,49 @@ def test_bake_and_strip_lora_on_float_and_quantized_bases(capsys):
     # a wrapper passed in directly comes back as its baked base
     top = LoRALinear.from_linear(torch.nn.Linear(8, 4, dtype=torch.float32), r=2)
     assert type(bake_and_strip_lora(top)) is torch.nn.Linear
+
+
+def test_save_model_bakes_and_strips_lora_wrappers(tmp_path):
+    """A model still wrapped in LoRA layers is saved as its baked base model
+    (model_saver.py:38-41 calls LoRASaver.bake_and_strip_lora first), so the
+    saved keys are the base model's and a fresh model reloads them all."""
+    from mflux_amd.lora import LoRALinear
+
+    torch.manual_seed(3)
+    pipe = Pipeline()
+    x = torch.randn(3, pipe.transformer.x_embedder.in_features)
+    pipe.transformer.x_embedder = LoRALinear.from_linear(pipe.transformer.x_embedder, r=4, scale=0.7)
+    with torch.no_grad():
+        pipe.transformer.x_embedder.lora_B.normal_()
+    want = pipe.transformer.x_embedder(x)
+    W.save_model(pipe, None, tmp_path, Definition)
+    assert type(pipe.transformer.x_embedder) is qnn.Linear           # stripped in place, as the reference does
+    index = json.load(open(tmp_path / "transformer" / "model.safetensors.index.json"))
+    assert "x_embedder.weight" in index["weight_map"]
+    assert not any("lora" in k or ".linear." in k for k in index["weight_map"])
+    fresh = Pipeline()
+    loaded = W.load_saved(Definition, tmp_path)
+    W.WeightApplier.apply_and_quantize(loaded, {"transformer": fresh.transformer, "vae": fresh.vae}, None, Definition)
+    assert torch.allclose(fresh.transformer.x_embedder(x), want, atol=1e-5)
+
+
+def test_update_module_writes_into_shared_storage():
+    """Layers stacked with concat_quantized(share_storage=True) are views of the
+    stack: loading stored tensors of the same shape afterwards must reach the
+    stack too (copied in place), not detach the layer from it."""
+    with qnn.placeholder_quantization():
+        a = qnn.QuantizedLinear(64, 8, bias=False, bits=4)
+        b = qnn.QuantizedLinear(64, 16, bias=False, bits=4)
+    model = torch.nn.ModuleDict({"a": a, "b": b})
+    stack = qnn.concat_quantized([a, b], share_storage=True)
+    new_w = torch.arange(16 * 8, dtype=torch.int32).reshape(16, 8).view(torch.uint32)
+    new_s = torch.full((16, 1), 0.5, dtype=b.scales.dtype)
+    done = W.update_module(model, {"b": {"weight": new_w, "scales": new_s}})
+    assert done == {"b.weight", "b.scales"}
+    assert torch.equal(stack.weight[8:].view(torch.int32), new_w.view(torch.int32))
+    assert torch.equal(stack.scales[8:], new_s)
+    assert b.weight.data_ptr() == stack.weight[8:].data_ptr()
+    # a value of another shape still replaces the tensor (a float weight becoming packed codes)
+    lin = torch.nn.ModuleDict({"l": qnn.Linear(64, 8, bias=False)})
+    W.update_module(lin, {"l": {"weight": torch.zeros(8, 8, dtype=torch.int32).view(torch.uint32)}})
+    assert lin["l"].weight.dtype == torch.uint32 and tuple(lin["l"].weight.shape) == (8, 8)

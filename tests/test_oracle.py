@@ -461,3 +461,16 @@ def test_silu_shape_properties(oracle):
     assert np.array_equal(y[big], x[big])
     order = np.argsort(x[x >= 0])
     assert np.all(np.diff(y[x >= 0][order]) >= 0)                          # monotone on the positive side
+
+
+def test_oracle_clean_under_host_sanitizers():
+    """`make -C oracle sanitize`: the C restatement under AddressSanitizer and
+    UndefinedBehaviorSanitizer on exactly-sized buffers, every entry point, all
+    storage types, bit widths and group sizes."""
+    import os
+    import subprocess
+
+    here = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+    res = subprocess.run(["make", "-C", here, "-B", "sanitize"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    assert "combinations clean" in res.stdout
