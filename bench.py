@@ -151,7 +151,7 @@ class Telemetry:
             "power_cap_w": int(cap) / 1e6 if cap else None,
             "sclk_mhz_mean": round(sum(mhz) / len(mhz), 1) if mhz else None,
             "sclk_mhz_min": min(mhz) if mhz else None,
-            "source": "sysfs hwmon power1 and pp_dpm_sclk of card 0, sampled every 10 ms over the timed region",
+            "source": "sysfs hwmon power1 and pp_dpm_sclk of card 0, sampled every 10 ms",
         }
 
 
@@ -237,6 +237,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sustain-s", type=float, default=1.5,
+                    help="seconds the step keeps running behind the timed region while socket power and "
+                         "shader clock are sampled (0: skip)")
     ap.add_argument("--cpu-sample-rows", type=int, default=2304)
     ap.add_argument("--no-secondary", action="store_true",
                     help="skip the GEMV and quantize measurements (they replay HIP graphs)")
@@ -301,18 +304,29 @@ def main():
             break
         prev = ms
     torch.cuda.synchronize()
-    with Telemetry() as telemetry:
-        t0 = time.perf_counter()
-        start = torch.cuda.Event(enable_timing=True)
-        stop = torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(args.steps):
-            step()
-        stop.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms_per_step = start.elapsed_time(stop) / args.steps
+    # The power sensor is a moving average that needs about half a second to follow the load, far
+    # longer than the timed region above: the same step therefore runs on for args.sustain_s
+    # seconds right behind it, and power and clock are the samples of the second half of that leg.
+    sustained = None
+    if args.sustain_s > 0:
+        n_sus = max(10, int(args.sustain_s * 1e3 / kernel_ms_per_step))
+        with Telemetry() as telemetry:
+            ms = event_ms(step, n_sus, torch)
+        telemetry.samples = telemetry.samples[len(telemetry.samples) // 2:]
+        sustained = {"steps": n_sus, "ms_per_step": round(ms, 4),
+                     "tflops": round(sum(2.0 * M_TOKENS * K * N for _, K, N in LINEARS) / ms / 1e9, 1),
+                     **telemetry.summary()}
 
     flops = sum(2.0 * M_TOKENS * K * N for _, K, N in LINEARS)
     value = flops / (ms_per_step * 1e-3) / 1e12
@@ -330,7 +344,7 @@ def main():
         "traffic_source": traffic_source,
         "avg_launch_us": round(kernel_ms_per_step * 1e3 / launches, 2),
         "flops_per_launch": flops / launches,
-        "telemetry": telemetry.summary(),
+        "sustained": sustained,
         "settling_ms_per_step": settle,
     }
 

@@ -147,6 +147,41 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
               int bits, void* y, int y_dtype, void* stream);
 
 /*
+ * mfq_qmm_t_ws with what the reference does to the linear's output next, done
+ * where the GEMM writes y (one pass over [M, N] instead of two to five
+ * element-wise ones).  `epilogue` is one of
+ *   MFQ_EPILOGUE_GELU           y = gelu_approx(linear(x)) for the columns from
+ *       act_from (a multiple of 8) on, linear(x) before them: the
+ *       nn.gelu_approx(self.proj_mlp(.)) of
+ *       src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53-54
+ *       (act_from > 0 when q, k, v and proj_mlp run as one stacked layer) and the
+ *       activation between the joint blocks' feed-forward linears (feed_forward.py:13-15);
+ *   MFQ_EPILOGUE_GATE_RESIDUAL  y = residual + gate * linear(x), gate [N] and
+ *       residual [M, N] in y's type, 16-byte aligned: residual + gate *
+ *       proj_out(.) of single_transformer_block.py:45,57 and hidden + gate *
+ *       ff(.) / gate * attn_output of joint_transformer_block.py:84-90;
+ *   MFQ_EPILOGUE_SWIGLU         y[M, N/2] = silu(g) * u, where the weight's rows
+ *       are the gate projection (w1) and the up projection (w3) in alternating
+ *       blocks of 32 rows (N % 64 == 0): nn.silu(self.w1(x)) * self.w3(x) of
+ *       src/mflux/models/z_image/model/z_image_transformer/feed_forward.py:13.
+ * x, scales, biases, bias and y share one 16-bit type.  Every step rounds to
+ * that type where the reference's separate operations would: the linear's
+ * output (and its bias add); gelu_approx once (MLX rounds inside it too:
+ * parity with MLX unpinned at that level); gate * y, then the sum with the
+ * residual; sigmoid, x * sigmoid, then the product with the up projection.
+ * MFQ_EUNSUPPORTED for M <= 16 (the matvec kernels have no epilogue), N % 8 != 0,
+ * and, with 256 x 256 tiles, shapes without whole scale periods (K/64 not a
+ * multiple of 4 * group_size / 64): run mfq_qmm_t and apply the operations.
+ * Unused pointer arguments are ignored; workspace as for mfq_qmm_t_ws.
+ */
+enum mfq_epilogue { MFQ_EPILOGUE_GELU = 1, MFQ_EPILOGUE_GATE_RESIDUAL = 2, MFQ_EPILOGUE_SWIGLU = 3 };
+int mfq_qmm_t_epilogue(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
+                       const void* scales, const void* biases, int sb_dtype, const void* bias,
+                       int64_t N, int group_size, int bits, int epilogue, const void* gate,
+                       const void* residual, int64_t act_from, void* y, int y_dtype, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+/*
  * y[m, k] = sum_n x[m, n] * (scales[n, k/gs] * code[n, k] + biases[n, k/gs]):
  * the product with the weight NOT transposed.  Replaces
  * mx.quantized_matmul(x, w, scales, biases, transpose=False, ...), which is the

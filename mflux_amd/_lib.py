@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmfq.so")
 
 F32, F16, BF16 = 0, 1, 2
 MFQ_EUNSUPPORTED = -8  # no kernel for this combination of arguments
+EPILOGUE_GELU, EPILOGUE_GATE_RESIDUAL, EPILOGUE_SWIGLU = 1, 2, 3
 MFQ_ESCRATCH = -9  # mfq_qmm_t_static: the K split needs more than the built-in buffer
 
 # every symbol include/mfq.h declares, with its ctypes signature
@@ -24,6 +25,8 @@ SIGNATURES = {
     "mfq_dequantize_affine": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_dequantize_rows": (_INT, [_PTR, _PTR, _PTR, _INT, _PTR, _I64, _I64, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmm_t_epilogue": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _INT, _PTR, _PTR,
+                                  _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),
     "mfq_qmm_n": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,

@@ -285,6 +285,90 @@ def silu_quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor
     return quantized_matmul(silu(x), w, scales, biases, transpose=True, group_size=group_size, bits=bits, mode=mode,
                             bias=bias)
 
+EPILOGUES = {"gelu": _lib.EPILOGUE_GELU, "gate_residual": _lib.EPILOGUE_GATE_RESIDUAL, "swiglu": _lib.EPILOGUE_SWIGLU}
+
+
+def gelu_approx(x: torch.Tensor) -> torch.Tensor:
+    """``nn.gelu_approx`` (the tanh form) evaluated in float32 and rounded once to
+    ``x``'s dtype, which is what the fused epilogue computes."""
+    return torch.nn.functional.gelu(x.float(), approximate="tanh").to(x.dtype)
+
+
+def swiglu_unstack(y: torch.Tensor) -> torch.Tensor:
+    """``silu(g) * u`` for ``y`` whose last axis holds gate and up values in
+    alternating blocks of 32 (the output of a layer made by ``nn.stack_gate_up``)."""
+    blocks = y.reshape(*y.shape[:-1], y.shape[-1] // 64, 2, 32)
+    return (silu(blocks[..., 0, :]) * blocks[..., 1, :]).reshape(*y.shape[:-1], y.shape[-1] // 2)
+
+
+def quantized_matmul_epilogue(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, *,
+                              epilogue: str, group_size: int = 64, bits: int = 4, mode: str = "affine",
+                              bias: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+                              residual: torch.Tensor | None = None, act_from: int = 0) -> torch.Tensor:
+    """A quantized linear and what the reference does to its output next, as one
+    kernel where a GEMM kernel runs (more than 16 rows of 16-bit ``x``); any other
+    call runs :func:`quantized_matmul` and the same operations on its result.
+
+    ``epilogue``:
+      ``"gelu"``           ``gelu_approx(linear(x))`` on the columns from ``act_from``
+                           (a multiple of 8) on: ``nn.gelu_approx(self.proj_mlp(.))``,
+                           src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53-54;
+      ``"gate_residual"``  ``residual + gate * linear(x)`` with ``gate`` of shape
+                           ``[N]`` (or ``[1, N]``) and ``residual`` of the output's
+                           shape: single_transformer_block.py:45,57,
+                           joint_transformer_block.py:84-90;
+      ``"swiglu"``         ``silu(g) * u`` for a weight whose rows alternate between
+                           the gate and the up projection in blocks of 32
+                           (``nn.stack_gate_up``); the result has ``N / 2`` columns:
+                           src/mflux/models/z_image/model/z_image_transformer/feed_forward.py:13.
+    Every step rounds to ``x``'s dtype as the separate operations do.  Inference
+    only (no autograd through the fused form: with gradients enabled on an input
+    the composed form runs)."""
+    _check_mode("quantized_matmul", mode)
+    _check_group_bits("quantized_matmul", group_size, bits)
+    if epilogue not in EPILOGUES:
+        raise ValueError(f"[quantized_matmul] unknown epilogue '{epilogue}' (one of {sorted(EPILOGUES)})")
+    _check_packed("quantized_matmul", w, scales, biases, group_size, bits)
+    N = w.shape[0]
+    K = w.shape[-1] * 32 // bits
+    if epilogue == "gate_residual":
+        if gate is None or residual is None:
+            raise ValueError("[quantized_matmul] the gate_residual epilogue needs gate and residual")
+        if gate.numel() != N or tuple(residual.shape) != (*x.shape[:-1], N):
+            raise ValueError(f"[quantized_matmul] gate must hold {N} values and residual have shape "
+                             f"{(*x.shape[:-1], N)}; got {tuple(gate.shape)} and {tuple(residual.shape)}")
+    if epilogue == "swiglu" and N % 64:
+        raise ValueError(f"[quantized_matmul] the swiglu epilogue needs gate and up rows in blocks of 32 (N % 64 == 0), got N = {N}")
+    if epilogue == "gelu" and (act_from < 0 or act_from > N or act_from % 8):
+        raise ValueError(f"[quantized_matmul] act_from must be a multiple of 8 in [0, {N}], got {act_from}")
+    tensors = [t for t in (x, bias, gate, residual) if t is not None]
+    needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+    M = x.numel() // K if x.ndim >= 1 and x.shape[-1] == K else 0
+    fusable = (M > 16 and not needs_grad and w.ndim == 2 and x.dtype == scales.dtype
+               and x.dtype in (torch.bfloat16, torch.float16)
+               and all(t.dtype == x.dtype for t in tensors))
+    if fusable:
+        _require_hip("quantized_matmul", x, "x")
+        _require_hip("quantized_matmul", w, "w")
+        if bias is not None and bias.shape != (N,):
+            raise ValueError(f"[quantized_matmul] bias must have shape ({N},), got {tuple(bias.shape)}")
+        y, ok = _lib.ops().qmm_t_epilogue(
+            x.reshape(M, K).contiguous(), w.contiguous(), scales.contiguous(), biases.contiguous(),
+            None if bias is None else bias.contiguous(), group_size, bits, EPILOGUES[epilogue],
+            None if gate is None else gate.reshape(N).contiguous(),
+            None if residual is None else residual.reshape(M, N).contiguous(), act_from)
+        if ok:
+            return y.reshape(*x.shape[:-1], y.shape[-1])
+    y = quantized_matmul(x, w, scales, biases, transpose=True, group_size=group_size, bits=bits, mode=mode, bias=bias)
+    if epilogue == "gelu":
+        if act_from == 0:
+            return gelu_approx(y)
+        return torch.cat([y[..., :act_from], gelu_approx(y[..., act_from:])], dim=-1)
+    if epilogue == "gate_residual":
+        return residual + gate.reshape(N) * y
+    return swiglu_unstack(y)
+
+
 def _low_rank_operands(low_rank, lead: tuple, M: int, N: int, compute: torch.dtype):
     """Checks ``(t, bs)`` against the product's shape; returns them as contiguous
     ``[M, R]`` / ``[N, R]`` matrices in the compute dtype."""

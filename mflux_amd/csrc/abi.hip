@@ -173,6 +173,43 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
                          workspace_bytes, (hipStream_t)stream, low_rank);
 }
 
+int mfq_qmm_t_epilogue(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                       const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits,
+                       int epilogue, const void* gate, const void* residual, int64_t act_from, void* y, int y_dtype,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (epilogue != MFQ_EPILOGUE_GELU && epilogue != MFQ_EPILOGUE_GATE_RESIDUAL && epilogue != MFQ_EPILOGUE_SWIGLU)
+    return MFQ_ESHAPE;
+  if (!is16(x_dtype) || x_dtype != sb_dtype || y_dtype != sb_dtype) return MFQ_EDTYPE;
+  if (M <= 0 || N <= 0 || K <= 0 || K % group_size) return MFQ_ESHAPE;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
+  if (!mfq::aligned16(x) || !mfq::aligned16(wq) || !mfq::aligned16(y)) return MFQ_EALIGN;
+  mfq::Epilogue epi;
+  epi.kind = epilogue;
+  if (epilogue == MFQ_EPILOGUE_GELU) {
+    if (act_from < 0 || act_from > N || act_from % 8) return MFQ_ESHAPE;
+    epi.act_from = (int)act_from;
+  } else if (epilogue == MFQ_EPILOGUE_GATE_RESIDUAL) {
+    if (!gate || !residual) return MFQ_ENULL;
+    if (!mfq::aligned16(gate) || !mfq::aligned16(residual)) return MFQ_EALIGN;
+    epi.gate = static_cast<const uint16_t*>(gate);
+    epi.residual = static_cast<const uint16_t*>(residual);
+  } else if (N % 64) {
+    return MFQ_ESHAPE;  // gate and up projections alternate in blocks of 32 rows
+  }
+  // the matvec kernels (M <= 16) have no epilogue, nor have rows that are not whole 16-byte pieces
+  if (M <= 16 || N % 8) return MFQ_EUNSUPPORTED;
+  if (bits != 4 && bits != 8)
+    return mfq::launch_qmm_mid_stream(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                      workspace, workspace_bytes, (hipStream_t)stream, mfq::LowRank(), epi);
+  if (K % 64)
+    return mfq::launch_qmm_mid(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, nullptr, 0,
+                               (hipStream_t)stream, mfq::LowRank(), epi);
+  return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, workspace,
+                         workspace_bytes, (hipStream_t)stream, mfq::LowRank(), epi);
+}
+
 int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
               const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y, int y_dtype, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;

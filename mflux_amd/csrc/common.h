@@ -293,6 +293,16 @@ struct LowRank {
   int R = 0;
 };
 
+// What a GEMM does to its 16-bit results on their way to y (the arithmetic is in epilogue.h).
+enum EpilogueKind { kEpiNone = 0, kEpiGelu = 1, kEpiGateResidual = 2, kEpiSwiglu = 3 };
+
+struct Epilogue {
+  int kind = kEpiNone;
+  const uint16_t* gate = nullptr;      // [N], 16-bit T
+  const uint16_t* residual = nullptr;  // [M, N], 16-bit T
+  int act_from = 0;                    // kEpiGelu: first column the activation applies to (a multiple of 8)
+};
+
 // Entry points of the individual translation units (host side).
 int launch_quantize(const void* w, int dtype, int64_t rows, int64_t K, int gs, int bits, uint32_t* wq,
                     void* scales, void* biases, hipStream_t stream);
@@ -327,24 +337,32 @@ int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32
 // adds it after the matvec kernels)
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
+               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank(),
+               Epilogue epi = Epilogue());
+// the instantiations of the same kernel with an epilogue (16-bit y, N % 8 == 0, period-wise scale loads;
+// MFQ_EUNSUPPORTED otherwise)
+int launch_qmm_epilogue(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                        const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                        void* workspace, size_t workspace_bytes, hipStream_t stream, Epilogue epi);
 // y[M, N] += t @ bs^T, rounded to y's type (dtype: the type of t, bs and a 16-bit y)
 int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream);
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // the 128-column-tile kernel for a few hundred activation rows, and for any M when K % 64 == 32
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
+                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank(),
+                   Epilogue epi = Epilogue());
 size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // the same kernel for 3, 5 and 6 bits (any M above one row; K % 32 == 0)
 int launch_qmm_mid_stream(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                           const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank());
+                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank = LowRank(),
+                          Epilogue epi = Epilogue());
 // y[M, K] = x[M, N] @ dequantize(wq[N, K]): the weight not transposed (N % 8 == 0)
 int launch_qmm_n(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
                  const void* biases, int64_t K, int gs, int bits, void* y, int y_dtype, hipStream_t stream);
 // y = sum of `splits` float32 planes of M x N (+ bias), rounded to y's type; dtype is the type of bias and 16-bit y
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
-                         int y_dtype, hipStream_t stream);
+                         int y_dtype, hipStream_t stream, Epilogue epi = Epilogue());
 
 }  // namespace mfq

@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "epilogue.h"
 
 namespace mfq {
 namespace {
@@ -149,12 +150,14 @@ __host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, 
   n0 = (in_band / band_rows) * BN;
 }
 
-template <typename T, int GS, int BITS, bool kFast, bool kLowRank>
+// kEpi: the tile's 16-bit results pass through `epi` (epilogue.h) on their way from the staging
+// region to y; instantiated apart so that the plain kernel's code is what it was.
+template <typename T, int GS, int BITS, bool kFast, bool kLowRank, bool kEpi>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void qmm_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
     int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits, float* __restrict__ planes,
-    const uint16_t* __restrict__ lr_t, const uint16_t* __restrict__ lr_bs, int lr_rank) {
+    const uint16_t* __restrict__ lr_t, const uint16_t* __restrict__ lr_bs, int lr_rank, Epilogue epi) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   using WR = WeightRegs<T, GS, BITS>;
@@ -584,10 +587,63 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
       // read back row-wise: lane l takes 16 bytes (8 columns) of row 8*k + l/8
       const int cg = n0 + wn + 8 * (lane & 7);
+      if constexpr (kEpi) {
+        if (epi.kind == kEpiSwiglu) {
+          // the wavefront's 64 columns are 32 of the gate projection, then their 32 of the up projection:
+          // lane l takes 8 gate columns and the 8 up columns 32 further of row 16*k + l/4 and writes
+          // 8 of the tile's 128 output columns (yout / out_stride address the [M, N/2] result)
+          const int cq = lane & 3;
+          const int co = (wn >> 1) + 8 * cq;  // output column inside the tile
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int rl = 16 * k + (lane >> 2);
+            const u32x4 g = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * cq);
+            const u32x4 u = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 64 + 16 * cq);
+            u32x4 v;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = epi_swiglu_pair<T>(g[c], u[c]);
+            const int row = m0 + 128 * pass + rl;
+            if (row < M && n0 + wn + 8 * cq < N)
+              *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + co) = v;
+          }
+          continue;
+        }
+        if (epi.kind == kEpiGateResidual) {
+          u32x4 gate8 = {0u, 0u, 0u, 0u};
+          if (cg < N) gate8 = *reinterpret_cast<const u32x4*>(epi.gate + cg);
+          const uint16_t* res = epi.residual + (int64_t)m0 * N + cg;  // row m0 of this lane's columns
+#pragma unroll
+          for (int k4 = 0; k4 < 4; ++k4) {
+            u32x4 rv[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {  // four rows' residuals requested before the first is needed
+              const int rl = 8 * (4 * k4 + kk) + (lane >> 3);
+              const int row = min(m0 + 128 * pass + rl, M - 1);
+              rv[kk] = cg < N ? *reinterpret_cast<const u32x4*>(res + (int64_t)(row - m0) * N) : gate8;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+              const int rl = 8 * (4 * k4 + kk) + (lane >> 3);
+              u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+#pragma unroll
+              for (int c = 0; c < 4; ++c) v[c] = epi_gate_residual_pair<T>(v[c], gate8[c], rv[kk][c]);
+              const int row = m0 + 128 * pass + rl;
+              if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
+            }
+          }
+          continue;
+        }
+      }
 #pragma unroll
       for (int k = 0; k < 16; ++k) {
         const int rl = 8 * k + (lane >> 3);
-        const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+        u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+        if constexpr (kEpi) {
+          if (epi.kind == kEpiGelu && cg >= epi.act_from) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = epi_gelu_pair<T>(v[c]);
+          }
+        }
         const int row = m0 + 128 * pass + rl;
         if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
         if (k & 1) __builtin_amdgcn_sched_barrier(0);
@@ -668,6 +724,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     if (item.plane < 0) {
       out_base = static_cast<char*>(y) + ((size_t)m0 * N + n0) * (y_is_f32 ? 4 : 2);
       out_stride = N;
+      if constexpr (kEpi) {
+        if (epi.kind == kEpiSwiglu) {  // y is [M, N/2], 16-bit
+          out_base = static_cast<char*>(y) + ((size_t)m0 * (N / 2) + n0 / 2) * 2;
+          out_stride = N / 2;
+        }
+      }
       out_f32 = y_is_f32;
       out_bias = bias;
     } else {
@@ -797,61 +859,86 @@ inline TailPlan plan_tail(int64_t M, int64_t N, int64_t K, int period, int cus) 
 
 inline int period_of(int gs) { return 4 * gs / BK; }
 
+// y = sum of `splits` dense float32 planes of M x N (+ bias), through the epilogue: the second kernel of
+// the 128-column-tile GEMM's K split.
 template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ planes, int splits,
                                                             int64_t plane_elems, const uint16_t* __restrict__ bias,
-                                                            int N, void* __restrict__ y, int y_is_f32) {
+                                                            int N, void* __restrict__ y, int y_is_f32, Epilogue epi) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  // the value of the linear layer in column c: rounded, then the bias added and rounded again, as the fused
+  // epilogue does (float32 y: one float32 sum)
+  auto linear = [&](float v, int c) {
+    const float bv = bias ? T::to_f32(bias[c]) : 0.f;
+    if (y_is_f32) return v + bv;
+    const float h = round_to<T>(v);
+    return bias ? round_to<T>(h + bv) : h;
+  };
+  auto sum4 = [&](int64_t q) {
+    float4 sum = reinterpret_cast<const float4*>(planes)[q];
+    for (int sp = 1; sp < splits; ++sp) {
+      const float4 v = reinterpret_cast<const float4*>(planes + sp * plane_elems)[q];
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    return sum;
+  };
   // four consecutive outputs per thread when rows are a multiple of four long
   // (a quad then never straddles two rows), one otherwise
   if ((N & 3) == 0) {
     for (int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; q < plane_elems / 4; q += stride) {
-      float4 sum = reinterpret_cast<const float4*>(planes)[q];
-      for (int sp = 1; sp < splits; ++sp) {
-        const float4 v = reinterpret_cast<const float4*>(planes + sp * plane_elems)[q];
-        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
-      }
       const int col = (int)((q * 4) % N);
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bias) {
+      if (epi.kind == kEpiSwiglu && (col & 32)) continue;  // the up projection's columns are read by the gate's threads
+      const float4 sum = sum4(q);
+      float v[4] = {linear(sum.x, col), linear(sum.y, col + 1), linear(sum.z, col + 2), linear(sum.w, col + 3)};
+      if (epi.kind == kEpiSwiglu) {  // N % 64 == 0; y is [M, N/2]
+        const float4 ups = sum4(q + 8);
+        const float u[4] = {linear(ups.x, col + 32), linear(ups.y, col + 33), linear(ups.z, col + 34), linear(ups.w, col + 35)};
+        const int64_t row = (q * 4) / N;
+        uint2 pk;
+        pk.x = T::pack2(epi_swiglu<T>(v[0], u[0]), epi_swiglu<T>(v[1], u[1]));
+        pk.y = T::pack2(epi_swiglu<T>(v[2], u[2]), epi_swiglu<T>(v[3], u[3]));
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(y) + row * (N / 2) + (col >> 6) * 32 + (col & 31)) = pk;
+        continue;
+      }
+      if (epi.kind == kEpiGelu && col >= epi.act_from) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) bv[c] = T::to_f32(bias[col + c]);
+        for (int c = 0; c < 4; ++c) v[c] = epi_gelu<T>(v[c]);
+      }
+      if (epi.kind == kEpiGateResidual) {
+        const uint2 g = *reinterpret_cast<const uint2*>(epi.gate + col);
+        const uint2 r = reinterpret_cast<const uint2*>(epi.residual)[q];
+        v[0] = epi_gate_residual<T>(v[0], lo_f32<T>(g.x), lo_f32<T>(r.x));
+        v[1] = epi_gate_residual<T>(v[1], hi_f32<T>(g.x), hi_f32<T>(r.x));
+        v[2] = epi_gate_residual<T>(v[2], lo_f32<T>(g.y), lo_f32<T>(r.y));
+        v[3] = epi_gate_residual<T>(v[3], hi_f32<T>(g.y), hi_f32<T>(r.y));
       }
       if (y_is_f32) {
-        reinterpret_cast<float4*>(y)[q] = make_float4(sum.x + bv[0], sum.y + bv[1], sum.z + bv[2], sum.w + bv[3]);
-      } else {  // round, then add the bias and round again, as the fused epilogue does
-        uint2 pk;
-        pk.x = T::pack2(sum.x, sum.y);
-        pk.y = T::pack2(sum.z, sum.w);
-        if (bias) {
-          pk.x = T::pack2(lo_f32<T>(pk.x) + bv[0], hi_f32<T>(pk.x) + bv[1]);
-          pk.y = T::pack2(lo_f32<T>(pk.y) + bv[2], hi_f32<T>(pk.y) + bv[3]);
-        }
-        reinterpret_cast<uint2*>(y)[q] = pk;
+        reinterpret_cast<float4*>(y)[q] = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+        reinterpret_cast<uint2*>(y)[q] = make_uint2(T::pack2(v[0], v[1]), T::pack2(v[2], v[3]));
       }
     }
-  } else {
+  } else {  // no epilogue on this path (the launcher refuses it)
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < plane_elems; i += stride) {
       float sum = planes[i];
       for (int sp = 1; sp < splits; ++sp) sum += planes[sp * plane_elems + i];
-      const float bv = bias ? T::to_f32(bias[i % N]) : 0.f;
+      const float v = linear(sum, (int)(i % N));
       if (y_is_f32) {
-        reinterpret_cast<float*>(y)[i] = sum + bv;
+        reinterpret_cast<float*>(y)[i] = v;
       } else {
-        uint16_t hv = T::from_f32(sum);
-        if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
-        reinterpret_cast<uint16_t*>(y)[i] = hv;
+        reinterpret_cast<uint16_t*>(y)[i] = T::from_f32(v);
       }
     }
   }
 }
 
-// y tile = sum of the `splits` planes of each tail tile (+ bias).  One thread per
+// y tile = sum of the `splits` planes of each tail tile (+ bias), through the epilogue.  One thread per
 // four consecutive columns of a tile row.
 template <typename T>
 __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restrict__ planes, int n_whole, int splits,
                                                           int tiles_m, int tiles_n, const uint16_t* __restrict__ bias,
-                                                          int M, int N, void* __restrict__ y, int y_is_f32) {
+                                                          int M, int N, void* __restrict__ y, int y_is_f32,
+                                                          Epilogue epi) {
   const int tail_tile = blockIdx.x / (BM * BN / 4 / 256);
   const int q = (blockIdx.x % (BM * BN / 4 / 256)) * 256 + threadIdx.x;  // quad inside the tile
   const int r = q / (BN / 4), c = (q % (BN / 4)) * 4;
@@ -859,33 +946,55 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
   tile_origin(n_whole + tail_tile, tiles_m, tiles_n, m0, n0);
   const int row = m0 + r, col = n0 + c;
   if (row >= M || col >= N) return;
+  if (epi.kind == kEpiSwiglu && (c & 32)) return;  // the up projection's columns are read by the gate's threads
   const float* src = planes + (size_t)tail_tile * splits * (BM * BN) + r * BN + c;
-  float4 sum = *reinterpret_cast<const float4*>(src);
-  for (int sp = 1; sp < splits; ++sp) {
-    const float4 v = *reinterpret_cast<const float4*>(src + (size_t)sp * (BM * BN));
-    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  auto sum_at = [&](const float* p) {
+    float4 sum = *reinterpret_cast<const float4*>(p);
+    for (int sp = 1; sp < splits; ++sp) {
+      const float4 v = *reinterpret_cast<const float4*>(p + (size_t)sp * (BM * BN));
+      sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    return sum;
+  };
+  // the value of the linear layer in column cc: rounded, then the bias added and rounded again, as the fused
+  // epilogue does (float32 y: one float32 sum)
+  auto linear = [&](float v, int cc) {
+    const float bv = bias ? T::to_f32(bias[cc]) : 0.f;
+    if (y_is_f32) return v + bv;
+    const float h = round_to<T>(v);
+    return bias ? round_to<T>(h + bv) : h;
+  };
+  const float4 sum = sum_at(src);
+  const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+  if (epi.kind == kEpiSwiglu) {
+    const float4 ups = sum_at(src + 32);
+    const float u[4] = {ups.x, ups.y, ups.z, ups.w};
+    uint16_t* dst = reinterpret_cast<uint16_t*>(y) + (int64_t)row * (N / 2) + (col >> 6) * 32 + (col & 31);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[e] = T::from_f32(epi_swiglu<T>(linear(v[e], col + e), linear(u[e], col + 32 + e)));
+    return;
   }
-  float v[4] = {sum.x, sum.y, sum.z, sum.w};
   const int64_t o = (int64_t)row * N + col;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     if (col + e >= N) break;
-    const float bv = bias ? T::to_f32(bias[col + e]) : 0.f;
+    float out = linear(v[e], col + e);
+    if (epi.kind == kEpiGelu && col + e >= epi.act_from) out = epi_gelu<T>(out);
+    if (epi.kind == kEpiGateResidual)
+      out = epi_gate_residual<T>(out, T::to_f32(epi.gate[col + e]), T::to_f32(epi.residual[o + e]));
     if (y_is_f32) {
-      reinterpret_cast<float*>(y)[o + e] = v[e] + bv;
-    } else {  // round, then add the bias and round again, as the fused epilogue does
-      uint16_t hv = T::from_f32(v[e]);
-      if (bias) hv = T::from_f32(T::to_f32(hv) + bv);
-      reinterpret_cast<uint16_t*>(y)[o + e] = hv;
+      reinterpret_cast<float*>(y)[o + e] = out;
+    } else {
+      reinterpret_cast<uint16_t*>(y)[o + e] = T::from_f32(out);
     }
   }
 }
 
-template <typename T, int GS, int BITS, bool kFast, bool kLowRank = false>
+template <typename T, int GS, int BITS, bool kFast, bool kLowRank = false, bool kEpi = false>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                   const void* bias, int64_t N, void* y, int y_dtype, TailPlan plan, void* planes, hipStream_t stream,
-                  LowRank lr = LowRank()) {
-  auto kernel = qmm_kernel<T, GS, BITS, kFast, kLowRank>;
+                  LowRank lr = LowRank(), Epilogue epi = Epilogue()) {
+  auto kernel = qmm_kernel<T, GS, BITS, kFast, kLowRank, kEpi>;
   static PerDeviceInt configured;
   if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
@@ -896,13 +1005,13 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
                      (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.n_whole, plan.splits,
-                     (float*)planes, (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R);
+                     (float*)planes, (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R, epi);
   if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
   if (plan.splits > 1) {
     const unsigned blocks = (unsigned)n_tail * (BM * BN / 4 / 256);
     hipLaunchKernelGGL((tail_reduce_kernel<T>), dim3(blocks), dim3(256), 0, stream, (const float*)planes, plan.n_whole,
                        plan.splits, tiles_m, tiles_n, (const uint16_t*)bias, (int)M, (int)N, y,
-                       (int)(y_dtype == MFQ_F32));
+                       (int)(y_dtype == MFQ_F32), epi);
     if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
   }
   return MFQ_OK;
@@ -916,7 +1025,7 @@ inline size_t tail_plane_bytes(int64_t M, int64_t N, TailPlan plan) {
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
-               hipStream_t stream, LowRank lr) {
+               hipStream_t stream, LowRank lr, Epilogue epi) {
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if ((M + BM) * lr.R >= (int64_t)1 << 31 || (N + BN) * lr.R >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
@@ -927,50 +1036,83 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
   const int64_t steps = K / BK;
   constexpr int kPer = ScaleRegs<T, GS>::kPeriod;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
-  if (!(steps % kPer == 0 && steps >= 4 && aligned8)) {
+  const bool fast = steps % kPer == 0 && steps >= 4 && aligned8;
+  TailPlan plan = fast ? plan_tail(M, N, K, kPer, compute_units()) : whole;
+  if (plan.splits > 1 && (!workspace || workspace_bytes < tail_plane_bytes(M, N, plan) || !aligned16(workspace)))
+    plan = whole;
+#ifdef MFQ_QMM_EPI
+  // the epilogues live in the staged 16-bit store of the period-wise kernel (the launcher has checked y and N)
+  if (!fast || lr.R) return MFQ_EUNSUPPORTED;
+  return launch_kernel<T, GS, BITS, true, false, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan,
+                                                       workspace, stream, lr, epi);
+#else
+  if (!fast) {
     // the rare shapes without period-wise scale loads: the update comes from its own kernel
     const int rc =
         launch_kernel<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, whole, nullptr, stream);
     return rc ? rc : launch_low_rank_add(T::code, lr, M, N, y, y_dtype, stream);
   }
-  TailPlan plan = plan_tail(M, N, K, kPer, compute_units());
-  if (plan.splits > 1 && (!workspace || workspace_bytes < tail_plane_bytes(M, N, plan) || !aligned16(workspace)))
-    plan = whole;
   if (lr.R)
     return launch_kernel<T, GS, BITS, true, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, workspace,
                                                   stream, lr);
   return launch_kernel<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, workspace, stream);
+#endif
 }
 
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                 const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-                hipStream_t stream, LowRank lr) {
+                hipStream_t stream, LowRank lr, Epilogue epi) {
   if (bits == 4)
-    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
-  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
 }
 
 template <typename T>
 int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
               const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-              hipStream_t stream, LowRank lr) {
+              hipStream_t stream, LowRank lr, Epilogue epi) {
   switch (gs) {
     case 32:
-      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr, epi);
     case 64:
-      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr, epi);
     default:
-      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr,
+                                 epi);
   }
+}
+
+int launch_types(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                 const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                 void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank, Epilogue epi) {
+  if (dtype == MFQ_BF16)
+    return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                           stream, low_rank, epi);
+  if (dtype == MFQ_F16)
+    return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                          stream, low_rank, epi);
+  return MFQ_EDTYPE;
 }
 
 }  // namespace
 
+// This file is compiled twice: as it is, and through qmm_epi.hip (which defines
+// MFQ_QMM_EPI and includes it) for the instantiations whose tiles pass through an
+// epilogue, so that the two sets build in parallel.
+#ifdef MFQ_QMM_EPI
+int launch_qmm_epilogue(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                        const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                        void* workspace, size_t workspace_bytes, hipStream_t stream, Epilogue epi) {
+  if (y_dtype == MFQ_F32 || N % 8) return MFQ_EUNSUPPORTED;  // the epilogues live in the 16-bit staged store
+  return launch_types(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                      stream, LowRank(), epi);
+}
+#else
 // Shapes whose 256 x 256 tiles would leave more than half of the compute units
 // idle go to the 128-column-tile kernel, except many rows against a long K,
 // where cutting K between 256 x 256 tiles measures about a tenth faster.
-inline bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
+bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
   const bool few_tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN) * 2 <= compute_units();
   return few_tiles && !(M > 512 && K >= 8192);
 }
@@ -982,7 +1124,7 @@ size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
 }
 
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
-                         int y_dtype, hipStream_t stream) {
+                         int y_dtype, hipStream_t stream, Epilogue epi) {
   const int64_t plane = M * N;
   const int64_t threads = (N & 3) == 0 ? plane / 4 : plane;
   const int64_t blocks = (threads + 255) / 256;
@@ -990,10 +1132,10 @@ int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, i
   const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
   if (dtype == MFQ_BF16) {
     hipLaunchKernelGGL((splitk_reduce_kernel<BF16>), grid, dim3(256), 0, stream, (const float*)planes, splits, plane,
-                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32));
+                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32), epi);
   } else if (dtype == MFQ_F16) {
     hipLaunchKernelGGL((splitk_reduce_kernel<F16>), grid, dim3(256), 0, stream, (const float*)planes, splits, plane,
-                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32));
+                       (const uint16_t*)bias, (int)N, y, (int)(y_dtype == MFQ_F32), epi);
   } else {
     return MFQ_EDTYPE;
   }
@@ -1002,17 +1144,16 @@ int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, i
 
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+               void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank, Epilogue epi) {
   if (use_mid_kernel(M, N, K))
     return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
-                          workspace_bytes, stream, low_rank);
-  if (dtype == MFQ_BF16)
-    return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                           stream, low_rank);
-  if (dtype == MFQ_F16)
-    return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                          stream, low_rank);
-  return MFQ_EDTYPE;
+                          workspace_bytes, stream, low_rank, epi);
+  if (epi.kind != kEpiNone)
+    return launch_qmm_epilogue(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
+                               workspace_bytes, stream, epi);
+  return launch_types(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
+                      stream, low_rank, epi);
 }
+#endif
 
 }  // namespace mfq

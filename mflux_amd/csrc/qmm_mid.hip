@@ -67,7 +67,7 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
     const uint16_t* __restrict__ x, const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
     const uint16_t* __restrict__ biases, const uint16_t* __restrict__ bias, void* __restrict__ y, int y_is_f32, int M,
     int N, int K, int tiles_m, int tiles_n, int steps, const uint16_t* __restrict__ lr_t,
-    const uint16_t* __restrict__ lr_bs, int lr_rank) {
+    const uint16_t* __restrict__ lr_bs, int lr_rank, Epilogue epi) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   constexpr int TM = tile_m(kWavesM);
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(threads_of(kWavesM), 2) void qmm_mid_kernel(
   }
 
   // ---- epilogue: every LDS tile is free now (the loop ended with a barrier)
-  store_block_64x64<T>(acc, lds, wave, lane, m0 + 64 * wm, n0 + 64 * wn, M, N, bias, y_item, y_is_f32);
+  store_block_64x64<T>(acc, lds, wave, lane, m0 + 64 * wm, n0 + 64 * wn, M, N, bias, y_item, y_is_f32, epi);
 }
 
 struct MidPlan {
@@ -380,7 +380,8 @@ inline MidPlan plan_mid(int64_t M, int64_t N, int64_t K, int period, int cus) {
 
 template <typename T, int GS, int BITS, bool kFast, int kWavesM>
 int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                  const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr) {
+                  const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr,
+                  Epilogue epi) {
   auto kernel = qmm_mid_kernel<T, GS, BITS, kFast, kWavesM>;
   constexpr int kLds = lds_bytes(kWavesM);
   static PerDeviceInt configured;
@@ -391,37 +392,39 @@ int launch_kernel(const void* x, int64_t M, int64_t K, const uint32_t* wq, const
   hipLaunchKernelGGL(kernel, dim3((unsigned)n_items), dim3(threads_of(kWavesM)), kLds, stream, (const uint16_t*)x, wq,
                      (const uint16_t*)scales, (const uint16_t*)biases, (const uint16_t*)bias, y,
                      (int)(y_dtype == MFQ_F32), (int)M, (int)N, (int)K, tiles_m, tiles_n, plan.steps,
-                     (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R);
+                     (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R, epi);
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 template <typename T, int GS, int BITS, bool kFast>
 int launch_tile(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr) {
+                const void* bias, int64_t N, void* y, int y_dtype, MidPlan plan, hipStream_t stream, LowRank lr,
+                Epilogue epi) {
   if (waves_m_of(M) == 2)
-    return launch_kernel<T, GS, BITS, kFast, 2>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr);
-  return launch_kernel<T, GS, BITS, kFast, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr);
+    return launch_kernel<T, GS, BITS, kFast, 2>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr, epi);
+  return launch_kernel<T, GS, BITS, kFast, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, plan, stream, lr, epi);
 }
 
 template <typename T, int GS, int BITS>
 int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                const void* bias, int64_t N, void* y, int y_dtype, void* workspace, size_t workspace_bytes,
-               hipStream_t stream, LowRank lr) {
+               hipStream_t stream, LowRank lr, Epilogue epi) {
   const int64_t steps = (K + TK - 1) / TK;
   constexpr int kPer = 4 * GS / TK;
   const bool aligned8 = ((reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases)) & 7u) == 0;
   if (!(K % TK == 0 && steps % kPer == 0 && aligned8))
     return launch_tile<T, GS, BITS, false>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
-                                           stream, lr);
+                                           stream, lr, epi);
   const MidPlan plan = plan_mid(M, N, K, kPer, compute_units());
   const size_t need = (size_t)plan.splits * M * N * sizeof(float);
   if (plan.splits == 1 || !workspace || workspace_bytes < need || !aligned16(workspace))
     return launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, MidPlan{1, (int)steps},
-                                          stream, lr);
+                                          stream, lr, epi);
+  // K cut into ranges: float32 planes, and the second kernel applies bias and epilogue
   if (int rc = launch_tile<T, GS, BITS, true>(x, M, K, wq, scales, biases, nullptr, N, workspace, MFQ_F32, plan,
-                                              stream, lr))
+                                              stream, lr, Epilogue()))
     return rc;
-  return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream);
+  return launch_splitk_reduce(T::code, workspace, plan.splits, M, N, bias, y, y_dtype, stream, epi);
 }
 
 // This file is compiled twice: as it is for 4 and 8 bits, and through
@@ -430,31 +433,31 @@ int launch_one(const void* x, int64_t M, int64_t K, const uint32_t* wq, const vo
 template <typename T, int GS>
 int launch_bits(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                 const void* bias, int64_t N, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-                hipStream_t stream, LowRank lr) {
+                hipStream_t stream, LowRank lr, Epilogue epi) {
 #ifdef MFQ_MID_STREAM
   if (bits == 3)
-    return launch_one<T, GS, 3>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+    return launch_one<T, GS, 3>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
   if (bits == 5)
-    return launch_one<T, GS, 5>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
-  return launch_one<T, GS, 6>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+    return launch_one<T, GS, 5>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
+  return launch_one<T, GS, 6>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
 #else
   if (bits == 4)
-    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
-  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr);
+    return launch_one<T, GS, 4>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
+  return launch_one<T, GS, 8>(x, M, K, wq, scales, biases, bias, N, y, y_dtype, ws, ws_bytes, stream, lr, epi);
 #endif
 }
 
 template <typename T>
 int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
               const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype, void* ws, size_t ws_bytes,
-              hipStream_t stream, LowRank lr) {
+              hipStream_t stream, LowRank lr, Epilogue epi) {
   switch (gs) {
     case 32:
-      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 32>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr, epi);
     case 64:
-      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 64>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr, epi);
     default:
-      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr);
+      return launch_bits<T, 128>(x, M, K, wq, scales, biases, bias, N, bits, y, y_dtype, ws, ws_bytes, stream, lr, epi);
   }
 }
 
@@ -463,7 +466,8 @@ int launch_gs(const void* x, int64_t M, int64_t K, const uint32_t* wq, const voi
 #ifdef MFQ_MID_STREAM
 int launch_qmm_mid_stream(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                           const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+                          void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank,
+                          Epilogue epi) {
 #else
 size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
   const MidPlan plan = plan_mid(M, N, K, period_of(gs), compute_units());
@@ -472,19 +476,21 @@ size_t qmm_mid_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
 
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
-                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank) {
+                   void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank, Epilogue epi) {
   if (bits != 4 && bits != 8)
     return launch_qmm_mid_stream(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
-                                 workspace_bytes, stream, low_rank);
+                                 workspace_bytes, stream, low_rank, epi);
 #endif
+  // an epilogue lives in the 16-bit staged store (and in the second kernel of a K split)
+  if (epi.kind != kEpiNone && (y_dtype == MFQ_F32 || N % 8)) return MFQ_EUNSUPPORTED;
   // 32-bit byte offsets into x, the packed weight and the scales
   if (M * K >= (int64_t)1 << 31 || N * K >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if (dtype == MFQ_BF16)
     return launch_gs<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                           stream, low_rank);
+                           stream, low_rank, epi);
   if (dtype == MFQ_F16)
     return launch_gs<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace, workspace_bytes,
-                          stream, low_rank);
+                          stream, low_rank, epi);
   return MFQ_EDTYPE;
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "common.h"
+#include "epilogue.h"
 
 namespace mfq {
 
@@ -14,10 +15,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // each wavefront transposes its block through a private region of it so that a
 // global store instruction writes whole row segments.  bias: [N] or nullptr,
 // added after the product has been rounded to T (two roundings, as a separate
-// add on the 16-bit result would do).
+// add on the 16-bit result would do).  epi (epilogue.h): applied to the 16-bit
+// results on their way from the staging region to y (16-bit y with N % 8 == 0
+// only: the launchers refuse an epilogue otherwise); for kEpiSwiglu y is [M, N/2].
 template <typename T>
 __device__ inline void store_block_64x64(const f32x16 (&acc)[2][2], char* lds, int wave, int lane, int mw, int nw, int M,
-                                         int N, const uint16_t* __restrict__ bias, char* y_item, int y_is_f32) {
+                                         int N, const uint16_t* __restrict__ bias, char* y_item, int y_is_f32,
+                                         const Epilogue epi = Epilogue()) {
   const int r = lane & 31;
   const int h = lane >> 5;
   if (!y_is_f32 && (N & 7) == 0) {
@@ -48,12 +52,41 @@ __device__ inline void store_block_64x64(const f32x16 (&acc)[2][2], char* lds, i
       }
     }
     const int cg = nw + 8 * (lane & 7);
+    if (epi.kind == kEpiSwiglu) {
+      // the block's 64 columns are 32 of the gate projection, then their 32 of the up projection: lane l
+      // takes 8 gate columns and the 8 up columns 32 further of row 16*k + l/4
+      const int cq = lane & 3;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int rl = 16 * k + (lane >> 2);
+        const u32x4 g = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 16 * cq);
+        const u32x4 u = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 64 + 16 * cq);
+        u32x4 v;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] = epi_swiglu_pair<T>(g[c], u[c]);
+        const int row = mw + rl;
+        if (row < M && nw < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * (N / 2) + (nw >> 1) + 8 * cq) = v;
+      }
+      return;
+    }
+    u32x4 gate8 = {0u, 0u, 0u, 0u};
+    if (epi.kind == kEpiGateResidual && cg < N) gate8 = *reinterpret_cast<const u32x4*>(epi.gate + cg);
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int rl = 8 * k + (lane >> 3);
-      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 16 * (lane & 7));
+      u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStride + 16 * (lane & 7));
       const int row = mw + rl;
-      if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
+      if (row < M && cg < N) {
+        if (epi.kind == kEpiGelu && cg >= epi.act_from) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] = epi_gelu_pair<T>(v[c]);
+        } else if (epi.kind == kEpiGateResidual) {
+          const u32x4 res = *reinterpret_cast<const u32x4*>(epi.residual + (int64_t)row * N + cg);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] = epi_gate_residual_pair<T>(v[c], gate8[c], res[c]);
+        }
+        *reinterpret_cast<u32x4*>(yout + (int64_t)row * N + cg) = v;
+      }
     }
   } else if (y_is_f32 && (N & 3) == 0) {
     constexpr int kStride = 64 * 4 + 16;

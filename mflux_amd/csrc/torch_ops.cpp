@@ -151,6 +151,43 @@ std::tuple<Tensor, bool> qmm_t(const Tensor& x, const Tensor& wq, const Tensor& 
   return {y, true};
 }
 
+// qmm_t with an epilogue of include/mfq.h's mfq_qmm_t_epilogue (1: gelu_approx from column act_from on,
+// 2: residual + gate * y, 3: SwiGLU of gate / up rows stacked in blocks of 32, y is [M, N/2]); `ok` is false
+// (and y undefined) when no kernel fuses it for the shape
+std::tuple<Tensor, bool> qmm_t_epilogue(const Tensor& x, const Tensor& wq, const Tensor& scales, const Tensor& biases,
+                                        const c10::optional<Tensor>& bias, int64_t group_size, int64_t bits,
+                                        int64_t epilogue, const c10::optional<Tensor>& gate,
+                                        const c10::optional<Tensor>& residual, int64_t act_from) {
+  const Matmul m = check_matmul("mfq::qmm_t_epilogue", x, wq, scales, biases, bias, bits);
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  const void *gate_p = nullptr, *res_p = nullptr;
+  if (epilogue == MFQ_EPILOGUE_GATE_RESIDUAL) {
+    TORCH_CHECK(gate.has_value() && residual.has_value(), "mfq::qmm_t_epilogue: gate and residual are required");
+    TORCH_CHECK(gate->dim() == 1 && gate->size(0) == m.N && gate->scalar_type() == x.scalar_type() &&
+                    gate->is_contiguous() && gate->device() == x.device(),
+                "mfq::qmm_t_epilogue: gate must be a contiguous [N] vector of x's dtype");
+    TORCH_CHECK(residual->dim() == 2 && residual->size(0) == m.M && residual->size(1) == m.N &&
+                    residual->scalar_type() == x.scalar_type() && residual->is_contiguous() &&
+                    residual->device() == x.device(),
+                "mfq::qmm_t_epilogue: residual must be a contiguous [M, N] matrix of x's dtype");
+    gate_p = gate->data_ptr();
+    res_p = residual->data_ptr();
+  }
+  const int64_t n_out = epilogue == MFQ_EPILOGUE_SWIGLU ? m.N / 2 : m.N;
+  Tensor y = at::empty({m.M, n_out}, x.options());
+  if (m.M == 0) return {y, true};
+  const size_t ws_bytes = mfq_qmm_t_workspace_bytes(m.M, m.K, m.N, (int)group_size, (int)bits);
+  Tensor ws;
+  if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  const int rc = mfq_qmm_t_epilogue(x.data_ptr(), m.sb, m.M, m.K, static_cast<const uint32_t*>(wq.data_ptr()),
+                                    scales.data_ptr(), biases.data_ptr(), m.sb, m.bias, m.N, (int)group_size,
+                                    (int)bits, (int)epilogue, gate_p, res_p, act_from, y.data_ptr(), m.sb,
+                                    ws_bytes ? ws.data_ptr() : nullptr, ws_bytes, stream_of(x));
+  if (rc == MFQ_EUNSUPPORTED) return {y, false};
+  check_status("mfq_qmm_t_epilogue", rc);
+  return {y, true};
+}
+
 // y[M, K] = x[M, N] @ dequantize(wq[N, K]); `ok` is false when N is not a multiple of 8
 std::tuple<Tensor, bool> qmm_n(const Tensor& x, const Tensor& wq, const Tensor& scales, const Tensor& biases,
                                int64_t group_size, int64_t bits, at::ScalarType out_dtype) {
@@ -205,6 +242,7 @@ TORCH_LIBRARY(mfq, m) {
   m.def("dequantize_affine(Tensor wq, Tensor scales, Tensor biases, int group_size, int bits, ScalarType out_dtype) -> Tensor");
   m.def("dequantize_rows(Tensor wq, Tensor scales, Tensor biases, Tensor indices, int group_size, int bits, ScalarType out_dtype) -> Tensor");
   m.def("qmm_t(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits, ScalarType out_dtype, Tensor? lr_t, Tensor? lr_bs) -> (Tensor, bool)");
+  m.def("qmm_t_epilogue(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits, int epilogue, Tensor? gate, Tensor? residual, int act_from) -> (Tensor, bool)");
   m.def("qmm_n(Tensor x, Tensor wq, Tensor scales, Tensor biases, int group_size, int bits, ScalarType out_dtype) -> (Tensor, bool)");
   m.def("qmv_silu(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits) -> (Tensor, bool)");
   m.def("low_rank_add_(Tensor(a!) y, Tensor t, Tensor bs) -> ()");
@@ -215,6 +253,7 @@ TORCH_LIBRARY_IMPL(mfq, CUDA, m) {  // the HIP backend answers to torch's CUDA d
   m.impl("dequantize_affine", dequantize_affine);
   m.impl("dequantize_rows", dequantize_rows);
   m.impl("qmm_t", qmm_t);
+  m.impl("qmm_t_epilogue", qmm_t_epilogue);
   m.impl("qmm_n", qmm_n);
   m.impl("qmv_silu", qmv_silu);
   m.impl("low_rank_add_", low_rank_add_);

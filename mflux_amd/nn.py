@@ -151,6 +151,90 @@ def silu_linear(layer: torch.nn.Module, x: torch.Tensor) -> torch.Tensor:
     return layer(core.silu(x))
 
 
+def _linear_parts(layer: torch.nn.Module, fn: str):
+    if not isinstance(layer, QuantizedLinear):
+        raise ValueError(f"[{fn}] expected a QuantizedLinear, got {type(layer).__name__}")
+    return layer.weight, layer.scales, layer.biases
+
+
+def gelu_linear(layer: torch.nn.Module, x: torch.Tensor, act_from: int = 0) -> torch.Tensor:
+    """``nn.gelu_approx(layer(x))`` as one kernel: the activation behind
+    ``proj_mlp`` of a single-stream block
+    (src/mflux/models/flux/model/flux_transformer/single_transformer_block.py:53-54)
+    and between the feed-forward linears of a joint block.  ``act_from``: the
+    first output column the activation applies to, for a layer that stacks q, k,
+    v and proj_mlp (``concat_quantized``) and activates only the last part.  A
+    float layer gets the composed form."""
+    if not isinstance(layer, QuantizedLinear):
+        y = layer(x)
+        return torch.cat([y[..., :act_from], core.gelu_approx(y[..., act_from:])], dim=-1) if act_from else core.gelu_approx(y)
+    w, s, b = _linear_parts(layer, "gelu_linear")
+    return core.quantized_matmul_epilogue(x, w, s, b, epilogue="gelu", group_size=layer.group_size, bits=layer.bits,
+                                          mode=layer.mode, bias=layer.bias, act_from=act_from)
+
+
+def gate_residual_linear(layer: torch.nn.Module, x: torch.Tensor, gate: torch.Tensor,
+                         residual: torch.Tensor) -> torch.Tensor:
+    """``residual + gate * layer(x)`` as one kernel, ``gate`` one value per output
+    feature (``[N]`` or ``[1, N]``): ``residual + gate * proj_out(.)`` of a
+    single-stream block (single_transformer_block.py:45,57) and ``hidden + gate *
+    ff(.)`` / ``hidden + gate * attn_output`` of a joint block
+    (joint_transformer_block.py:84-90).  A float layer gets the composed form."""
+    if not isinstance(layer, QuantizedLinear):
+        return residual + gate.reshape(-1) * layer(x)
+    w, s, b = _linear_parts(layer, "gate_residual_linear")
+    return core.quantized_matmul_epilogue(x, w, s, b, epilogue="gate_residual", group_size=layer.group_size,
+                                          bits=layer.bits, mode=layer.mode, bias=layer.bias, gate=gate,
+                                          residual=residual)
+
+
+def stack_gate_up(gate_layer: QuantizedLinear, up_layer: QuantizedLinear) -> QuantizedLinear:
+    """The gate (``w1``) and up (``w3``) projections of a SwiGLU feed-forward
+    (src/mflux/models/z_image/model/z_image_transformer/feed_forward.py:8-13) as
+    one ``QuantizedLinear`` whose rows alternate between the two in blocks of 32:
+    rows ``64 i .. 64 i + 31`` are rows ``32 i ..`` of the gate projection, the next
+    32 the same rows of the up projection.  A packed row belongs to its output
+    feature alone, so this is a permutation of rows of codes, scales and biases
+    and needs no requantization.  ``swiglu_linear`` evaluates ``silu(w1 x) * w3 x``
+    on it in one kernel: both values of an output land in the same register of
+    the same lane."""
+    for layer in (gate_layer, up_layer):
+        _linear_parts(layer, "stack_gate_up")
+    a, b = gate_layer, up_layer
+    if (a.input_dims, a.output_dims, a.group_size, a.bits, a.mode, a.scales.dtype) != (
+            b.input_dims, b.output_dims, b.group_size, b.bits, b.mode, b.scales.dtype):
+        raise ValueError("[stack_gate_up] the two layers must share shape, group_size, bits, mode and dtype")
+    if a.output_dims % 32:
+        raise ValueError(f"[stack_gate_up] output_dims must be a multiple of 32, got {a.output_dims}")
+    if (a.bias is None) != (b.bias is None):
+        raise ValueError("[stack_gate_up] both layers or neither must have a bias")
+
+    def weave(p, q):
+        return torch.stack([p.reshape(-1, 32, *p.shape[1:]), q.reshape(-1, 32, *q.shape[1:])], dim=1).reshape(
+            2 * p.shape[0], *p.shape[1:])
+
+    out = QuantizedLinear.__new__(QuantizedLinear)
+    torch.nn.Module.__init__(out)
+    out.group_size, out.bits, out.mode = a.group_size, a.bits, a.mode
+    out.register_buffer("weight", weave(a.weight.view(torch.int32), b.weight.view(torch.int32)).view(torch.uint32))
+    out.register_buffer("scales", weave(a.scales, b.scales))
+    out.register_buffer("biases", weave(a.biases, b.biases))
+    if a.bias is not None:
+        out.register_buffer("bias", weave(a.bias, b.bias))
+    else:
+        out.bias = None
+    return out
+
+
+def swiglu_linear(stacked: QuantizedLinear, x: torch.Tensor) -> torch.Tensor:
+    """``silu(w1 x) * w3 x`` for ``stacked = stack_gate_up(w1, w3)``: one GEMM over
+    both projections whose epilogue writes the ``[..., N / 2]`` product, instead
+    of two GEMMs and three element-wise passes."""
+    w, s, b = _linear_parts(stacked, "swiglu_linear")
+    return core.quantized_matmul_epilogue(x, w, s, b, epilogue="swiglu", group_size=stacked.group_size,
+                                          bits=stacked.bits, mode=stacked.mode, bias=stacked.bias)
+
+
 def concat_quantized(layers: list[QuantizedLinear], share_storage: bool = False) -> QuantizedLinear:
     """One ``QuantizedLinear`` whose output is the outputs of ``layers`` side by
     side: the packed rows, scales and biases of a weight belong to its output
