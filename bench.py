@@ -478,6 +478,52 @@ def main():
         ms = graph_ms(lambda: mflux_amd.quantized_matmul(xm, wqm, sm, bm, group_size=GS, bits=BITS), 10, 5, torch)
         medium[f"{Km}x{Nm}"] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * 512 * Km * Nm / ms / 1e9, 1)}
 
+    # ---- secondary: what follows the linear, inside the GEMM against element-wise passes behind it ----
+    #   single block: gelu_approx on proj_mlp's part of linear1 (columns from 9216 on), and
+    #   residual + gate * linear2(.) (single_transformer_block.py:45-57);
+    #   Z-Image: silu(w1 x) * w3 x at M = 4352, 3840 -> 2 x 10240, W8 (feed_forward.py:13).
+    fused = {}
+    if not args.no_secondary:
+        from mflux_amd import nn as qnn
+
+        def best_of(calls):
+            for fn in calls.values():
+                for _ in range(3):
+                    fn()
+            best = {key: float("inf") for key in calls}
+            for _ in range(3):
+                for key, fn in calls.items():
+                    best[key] = min(best[key], event_ms(fn, 10, torch))
+            return {key: round(ms * 1e3, 1) for key, ms in best.items()}
+
+        (_, x1, wq1, s1, b1), (_, x2, wq2, s2, b2) = ops
+        fused["linear1_gelu_from_9216"] = best_of({
+            "fused_us": lambda: mflux_amd.quantized_matmul_epilogue(x1, wq1, s1, b1, epilogue="gelu", group_size=GS,
+                                                                    bits=BITS, act_from=9216),
+            "separate_us": lambda: torch.cat([(y := mflux_amd.quantized_matmul(x1, wq1, s1, b1, group_size=GS, bits=BITS))[:, :9216],
+                                              mflux_amd.gelu_approx(y[:, 9216:])], dim=1),
+        })
+        gate = seeded_bf16(torch, dev, CONFIG, 30, (3072,), 1.0)
+        res = seeded_bf16(torch, dev, CONFIG, 31, (M_TOKENS, 3072), 1.0)
+        fused["linear2_gate_residual"] = best_of({
+            "fused_us": lambda: mflux_amd.quantized_matmul_epilogue(x2, wq2, s2, b2, epilogue="gate_residual",
+                                                                    group_size=GS, bits=BITS, gate=gate, residual=res),
+            "separate_us": lambda: res + gate * mflux_amd.quantized_matmul(x2, wq2, s2, b2, group_size=GS, bits=BITS),
+        })
+        del gate, res
+        xz = seeded_bf16(torch, dev, 4, 10, (4352, 3840), 1.0)
+        halves = []
+        for idx in (11, 21):
+            lin = qnn.QuantizedLinear(3840, 10240, bias=False, group_size=GS, bits=8)
+            lin.weight, lin.scales, lin.biases = mflux_amd.quantize(seeded_bf16(torch, dev, 4, idx, (10240, 3840), 0.02), GS, 8)
+            halves.append(lin)
+        stacked = qnn.stack_gate_up(*halves)
+        fused["zimage_swiglu_3840_to_2x10240_w8"] = best_of({
+            "fused_us": lambda: qnn.swiglu_linear(stacked, xz),
+            "separate_us": lambda: mflux_amd.silu(halves[0](xz)) * halves[1](xz),
+        })
+        del xz, halves, stacked
+
     quant = {}
     for (name, K, N) in (() if args.no_secondary else LINEARS):
         ms = quant_ms[name]
@@ -516,7 +562,8 @@ def main():
         "secondary": {"metric": "W8 GEMV GB/s (adaLN 3072->18432, cold weights)", "roofline": gemv_roofline,
                       "gemv_w8": gemv.get("w8", {}),
                       "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
-                      "qmm_w4_lora_r16": lora, "library_bf16_gemm_same_operands": library},
+                      "qmm_w4_lora_r16": lora, "epilogues_fused_vs_separate": fused,
+                      "library_bf16_gemm_same_operands": library},
     }
     if not args.no_cpu_baseline:
         name, x, wq, s, b = ops[0]
