@@ -523,6 +523,18 @@ def main():
             "separate_us": lambda: mflux_amd.silu(halves[0](xz)) * halves[1](xz),
         })
         del xz, halves, stacked
+        # the step in front of the modulated linears: LayerNorm(x) * (1 + scale) + shift over [4608, 3072]
+        xn = seeded_bf16(torch, dev, CONFIG, 40, (M_TOKENS, 3072), 1.0)
+        scn, shn = seeded_bf16(torch, dev, CONFIG, 41, (3072,), 0.3), seeded_bf16(torch, dev, CONFIG, 42, (3072,), 0.3)
+        # (10 us kernels: back to back in a HIP graph, as the matvecs are timed)
+        fused["layer_norm_modulate_4608x3072"] = {
+            "fused_us": round(graph_ms(lambda: mflux_amd.layer_norm_modulate(xn, scn, shn), 16, 5, torch) * 1e3, 2),
+            "separate_us": round(graph_ms(
+                lambda: torch.nn.functional.layer_norm(xn, (3072,), eps=1e-6) * (1 + scn) + shn, 16, 5, torch) * 1e3, 2),
+        }
+        fused["layer_norm_modulate_4608x3072"]["frac_hbm"] = round(
+            2 * 2 * M_TOKENS * 3072 / (fused["layer_norm_modulate_4608x3072"]["fused_us"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)
+        del xn, scn, shn
 
     quant = {}
     for (name, K, N) in (() if args.no_secondary else LINEARS):

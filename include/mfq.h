@@ -296,6 +296,28 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
                        size_t workspace_bytes, void* stream);
 
 /*
+ * y = LayerNorm(x, eps) * (1 + scale) + shift, row by row: the normalisation
+ * without learned parameters and the adaLN modulation in front of every
+ * modulated linear of the DiT blocks, four element-wise passes in the reference
+ *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:22
+ *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero_single.py:19
+ *   src/mflux/models/flux/model/flux_transformer/ada_layer_norm_continuous.py:21
+ *   src/mflux/models/flux/model/flux_transformer/joint_transformer_block.py:86-87
+ * (nn.LayerNorm(dims, eps=1e-6, affine=False), then * (1 + scale), + shift).
+ *   x, y    [M, K]                      dtype (MFQ_BF16 or MFQ_F16), 16-byte aligned
+ *   scale, shift  [M / rows_per_vector, K]  dtype, 16-byte aligned: one vector per
+ *                 batch entry, shared by rows_per_vector consecutive rows; both
+ *                 NULL for the plain LayerNorm (rows_per_vector is then ignored)
+ * Mean and variance are float32 sums over the row; the normalised value,
+ * 1 + scale, their product and the sum with the shift are each rounded to
+ * dtype, as the reference's separate operations on a 16-bit array round
+ * (the order of the float32 sums inside MLX's layer norm: parity unpinned).
+ * MFQ_EUNSUPPORTED for K > 8192 or K % 8 != 0.
+ */
+int mfq_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, const void* scale,
+                            const void* shift, int64_t rows_per_vector, float eps, void* y, void* stream);
+
+/*
  * y[M, N] += t[M, rank] @ bs[N, rank]^T in float32, rounded to y_dtype (dtype
  * or MFQ_F32): the same adapters (see mfq_qmm_t_low_rank for t and bs) behind
  * a product that did not come from mfq_qmm_t_low_rank, e.g. an odd bit width

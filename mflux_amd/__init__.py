@@ -3,9 +3,9 @@ linears, a drop-in for the MLX operations mflux's diffusion transformers run
 through (``mx.quantize`` / ``nn.quantize`` / ``QuantizedLinear`` /
 ``mx.quantized_matmul``)."""
 from . import lora, nn, weights
-from .core import (dequantize, dequantize_rows, gelu_approx, quantize, quantized_matmul, quantized_matmul_epilogue,
+from .core import (dequantize, dequantize_rows, gelu_approx, layer_norm_modulate, quantize, quantized_matmul, quantized_matmul_epilogue,
                    silu, silu_quantized_matmul)
 
 __all__ = ["nn", "lora", "weights", "quantize", "dequantize", "dequantize_rows", "quantized_matmul",
-           "quantized_matmul_epilogue", "silu", "gelu_approx", "silu_quantized_matmul"]
+           "quantized_matmul_epilogue", "silu", "gelu_approx", "silu_quantized_matmul", "layer_norm_modulate"]
 __version__ = "0.1.0"

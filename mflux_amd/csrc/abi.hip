@@ -242,6 +242,18 @@ int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
   return MFQ_EUNSUPPORTED;
 }
 
+int mfq_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, const void* scale, const void* shift,
+                            int64_t rows_per_vector, float eps, void* y, void* stream) {
+  if (!is16(dtype)) return MFQ_EDTYPE;
+  if (M <= 0 || K <= 0 || M > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!x || !y || (scale == nullptr) != (shift == nullptr)) return MFQ_ENULL;
+  if (scale && (rows_per_vector <= 0 || M % rows_per_vector)) return MFQ_ESHAPE;
+  if (!(eps >= 0.f)) return MFQ_ESHAPE;
+  if (!mfq::aligned16(x) || !mfq::aligned16(y) || !mfq::aligned16(scale) || !mfq::aligned16(shift)) return MFQ_EALIGN;
+  return mfq::launch_layer_norm_modulate(x, dtype, M, K, scale, shift, scale ? rows_per_vector : M, eps, y,
+                                         (hipStream_t)stream);
+}
+
 int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank, void* y, int y_dtype,
                      void* stream) {
   if (!is16(dtype)) return MFQ_EDTYPE;

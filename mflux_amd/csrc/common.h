@@ -361,6 +361,10 @@ int launch_qmm_mid_stream(const void* x, int dtype, int64_t M, int64_t K, const 
 // y[M, K] = x[M, N] @ dequantize(wq[N, K]): the weight not transposed (N % 8 == 0)
 int launch_qmm_n(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
                  const void* biases, int64_t K, int gs, int bits, void* y, int y_dtype, hipStream_t stream);
+// y = LayerNorm(x, eps) (* (1 + scale) + shift): rows of up to 8192 16-bit elements, K % 8 == 0; scale and shift
+// [M / rows_per_vector, K] or both nullptr
+int launch_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, const void* scale, const void* shift,
+                               int64_t rows_per_vector, float eps, void* y, hipStream_t stream);
 // y = sum of `splits` float32 planes of M x N (+ bias), rounded to y's type; dtype is the type of bias and 16-bit y
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
                          int y_dtype, hipStream_t stream, Epilogue epi = Epilogue());

@@ -223,6 +223,35 @@ std::tuple<Tensor, bool> qmv_silu(const Tensor& x, const Tensor& wq, const Tenso
   return {y, true};
 }
 
+// LayerNorm(x, eps) * (1 + scale) + shift over the rows of x [M, K]; scale and shift [B, K] with M % B == 0 (or
+// neither); `ok` is false when the rows are too long for the kernel
+std::tuple<Tensor, bool> layer_norm_modulate(const Tensor& x, const c10::optional<Tensor>& scale,
+                                             const c10::optional<Tensor>& shift, double eps) {
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "mfq::layer_norm_modulate: x must be a contiguous matrix");
+  TORCH_CHECK(scale.has_value() == shift.has_value(), "mfq::layer_norm_modulate: scale and shift come together");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  const int64_t M = x.size(0), K = x.size(1);
+  int64_t rows_per_vector = M;
+  const void *sc = nullptr, *sh = nullptr;
+  if (scale.has_value()) {
+    TORCH_CHECK(scale->dim() == 2 && scale->size(1) == K && scale->sizes() == shift->sizes() && scale->size(0) > 0 &&
+                    M % scale->size(0) == 0 && scale->scalar_type() == x.scalar_type() &&
+                    shift->scalar_type() == x.scalar_type() && scale->is_contiguous() && shift->is_contiguous() &&
+                    scale->device() == x.device() && shift->device() == x.device(),
+                "mfq::layer_norm_modulate: scale and shift must be contiguous [B, K] matrices of x's dtype, M % B == 0");
+    rows_per_vector = M / scale->size(0);
+    sc = scale->data_ptr();
+    sh = shift->data_ptr();
+  }
+  Tensor y = at::empty_like(x);
+  if (M == 0) return {y, true};
+  const int rc = mfq_layer_norm_modulate(x.data_ptr(), dtype_code(x.scalar_type(), "x"), M, K, sc, sh, rows_per_vector,
+                                         (float)eps, y.data_ptr(), stream_of(x));
+  if (rc == MFQ_EUNSUPPORTED) return {y, false};
+  check_status("mfq_layer_norm_modulate", rc);
+  return {y, true};
+}
+
 // y += t @ bs^T in place
 void low_rank_add_(Tensor& y, const Tensor& t, const Tensor& bs) {
   TORCH_CHECK(y.dim() == 2 && t.dim() == 2 && bs.dim() == 2 && y.is_contiguous() && t.is_contiguous() &&
@@ -245,6 +274,7 @@ TORCH_LIBRARY(mfq, m) {
   m.def("qmm_t_epilogue(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits, int epilogue, Tensor? gate, Tensor? residual, int act_from) -> (Tensor, bool)");
   m.def("qmm_n(Tensor x, Tensor wq, Tensor scales, Tensor biases, int group_size, int bits, ScalarType out_dtype) -> (Tensor, bool)");
   m.def("qmv_silu(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits) -> (Tensor, bool)");
+  m.def("layer_norm_modulate(Tensor x, Tensor? scale, Tensor? shift, float eps) -> (Tensor, bool)");
   m.def("low_rank_add_(Tensor(a!) y, Tensor t, Tensor bs) -> ()");
 }
 
@@ -256,5 +286,6 @@ TORCH_LIBRARY_IMPL(mfq, CUDA, m) {  // the HIP backend answers to torch's CUDA d
   m.impl("qmm_t_epilogue", qmm_t_epilogue);
   m.impl("qmm_n", qmm_n);
   m.impl("qmv_silu", qmv_silu);
+  m.impl("layer_norm_modulate", layer_norm_modulate);
   m.impl("low_rank_add_", low_rank_add_);
 }

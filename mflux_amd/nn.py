@@ -157,6 +157,14 @@ def _linear_parts(layer: torch.nn.Module, fn: str):
     return layer.weight, layer.scales, layer.biases
 
 
+def layer_norm_modulate(x: torch.Tensor, scale: torch.Tensor | None = None, shift: torch.Tensor | None = None,
+                        eps: float = 1e-6) -> torch.Tensor:
+    """``nn.LayerNorm(dims, eps, affine=False)(x) * (1 + scale) + shift`` as one
+    pass (``core.layer_norm_modulate``): the step in front of the modulated
+    linears, e.g. src/mflux/models/flux/model/flux_transformer/ada_layer_norm_zero.py:22."""
+    return core.layer_norm_modulate(x, scale, shift, eps)
+
+
 def gelu_linear(layer: torch.nn.Module, x: torch.Tensor, act_from: int = 0) -> torch.Tensor:
     """``nn.gelu_approx(layer(x))`` as one kernel: the activation behind
     ``proj_mlp`` of a single-stream block
