@@ -320,8 +320,8 @@ int mfq_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, cons
 /*
  * y[M, N] += t[M, rank] @ bs[N, rank]^T in float32, rounded to y_dtype (dtype
  * or MFQ_F32): the same adapters (see mfq_qmm_t_low_rank for t and bs) behind
- * a product that did not come from mfq_qmm_t_low_rank, e.g. an odd bit width
- * with M > 1 that the caller dequantized and multiplied with a library GEMM.
+ * a product that did not come from mfq_qmm_t_low_rank, e.g. one of the matvec
+ * kernels (M <= 16) or mfq_qmm_n.
  */
 int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank,
                      void* y, int y_dtype, void* stream);
