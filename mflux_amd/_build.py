@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libmfq.so")
-SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "lora.hip", "norm.hip")
+SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "qmm_frag.hip", "lora.hip", "norm.hip")
 
 # -ffp-contract=off, correctly rounded division and preserved denormals make
 # the quantize kernel's float32 arithmetic the same IEEE operations as the
@@ -42,10 +42,58 @@ def _compile(src: str) -> str:
     return obj
 
 
+# Kernels whose matrix instructions are inline assembly (result tied to the addend), which the compiler's
+# hazard recognizer cannot see: {source: substring of the kernels' mangled names}.
+ASM_MFMA_KERNELS = {"qmm_frag.hip": "frag_gemm_kernel"}
+
+
+def check_accumulator_moves(src: str) -> int:
+    """Compiles `src` to assembly (device side) and checks every kernel named in
+    ASM_MFMA_KERNELS: no basic block may hold both a matrix instruction and an
+    instruction that moves an accumulator between register files
+    (v_accvgpr_read / _write / _mov).  The kernels keep such moves (zeroing, the
+    epilogue's reads) in blocks of their own, behind wait states of their own;
+    one next to a matrix instruction would read or overwrite a result in flight
+    without the hardware or the compiler noticing.  Returns the number of kernels
+    checked; raises on a finding."""
+    import re
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        asm = os.path.join(tmp, "out.s")
+        cmd = [hipcc(), *HIPCC_FLAGS, "--cuda-device-only", "-S", "-c", os.path.join(CSRC, src), "-o", asm]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed on {src}:\n{res.stdout}\n{res.stderr}")
+        text = open(asm).read()
+    checked = 0
+    for m in re.finditer(r"^(\S*%s\S*):" % re.escape(ASM_MFMA_KERNELS[src]), text, re.M):
+        body = text[m.end():text.index(".Lfunc_end", m.end())]
+        n_matrix = 0
+        for block in re.split(r"\n\.LBB[0-9_]+:", body):
+            ops = [ln.split()[0] for ln in block.split("\n") if ln.strip() and not ln.strip().startswith((";", "."))]
+            matrix = sum(op.startswith("v_mfma") for op in ops)
+            moves = sum(op.startswith("v_accvgpr") for op in ops)
+            n_matrix += matrix
+            if matrix and moves:
+                raise RuntimeError(f"{src}: {m.group(1)} has a basic block with {matrix} matrix instructions and "
+                                   f"{moves} accumulator moves")
+        if not n_matrix:
+            raise RuntimeError(f"{src}: {m.group(1)} holds no matrix instruction; the check does not see the kernel")
+        checked += 1
+    if not checked:
+        raise RuntimeError(f"{src}: no kernel named *{ASM_MFMA_KERNELS[src]}* found")
+    return checked
+
+
 def build_library(verbose: bool = False) -> str:
-    """Always recompiles every translation unit and relinks libmfq.so."""
-    with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
+    """Always recompiles every translation unit, checks the generated code of the
+    kernels in ASM_MFMA_KERNELS and relinks libmfq.so."""
+    with ThreadPoolExecutor(max_workers=len(SOURCES) + len(ASM_MFMA_KERNELS)) as pool:
+        checks = [pool.submit(check_accumulator_moves, src) for src in ASM_MFMA_KERNELS]
         objs = list(pool.map(_compile, SOURCES))
+        for c in checks:
+            c.result()
     tmp = LIB_PATH + ".tmp"
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -96,7 +96,7 @@ size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size
   if (N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
   if (bits != 4 && bits != 8) return M > 1 ? mfq::qmm_mid_workspace_bytes(M, N, K, group_size) : 0;
   if (M <= 16) return 0;
-  return mfq::qmm_workspace_bytes(M, N, K, group_size);
+  return mfq::qmm_workspace_bytes(M, N, K, group_size, bits);
 }
 
 int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
@@ -117,7 +117,9 @@ int mfq_qmm_t_static(const void* x, int x_dtype, int64_t M, int64_t K, const uin
                      const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits, void* y,
                      int y_dtype, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
-  const size_t need = mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits);
+  size_t need = mfq_qmm_t_workspace_bytes(M, K, N, group_size, bits);
+  // a scratch copy of the weights that does not fit is done without (the fused kernel); the planes of a K split are not
+  if (need > kScratchBytes && (bits == 4 || bits == 8) && M > 16) need = mfq::qmm_min_workspace_bytes(M, N, K, group_size);
   if (need > kScratchBytes) return MFQ_ESCRATCH;
   void* ws = nullptr;
   if (need) {

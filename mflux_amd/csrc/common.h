@@ -346,7 +346,18 @@ int launch_qmm_epilogue(const void* x, int dtype, int64_t M, int64_t K, const ui
                         void* workspace, size_t workspace_bytes, hipStream_t stream, Epilogue epi);
 // y[M, N] += t @ bs^T, rounded to y's type (dtype: the type of t, bs and a 16-bit y)
 int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream);
-size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
+// what a caller should bring (the K split's planes, or the scratch copy of the two-kernel path where that is
+// preferred) and what the call cannot do without (the planes only)
+size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits);
+size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
+// the two-kernel path (qmm_frag.hip): dequantize once into a 16-bit copy in fragment order (workspace:
+// qmm_frag_workspace_bytes, 16-byte aligned), then a GEMM on 16x16x32 matrix instructions; 4 and 8 bits,
+// 16-bit y of x's type, epilogues as launch_qmm_epilogue
+bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits);
+size_t qmm_frag_workspace_bytes(int64_t N, int64_t K);
+int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
+                    hipStream_t stream, Epilogue epi);
 // the 128-column-tile kernel for a few hundred activation rows, and for any M when K % 64 == 32
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,

@@ -1117,10 +1117,29 @@ bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
   return few_tiles && !(M > 512 && K >= 8192);
 }
 
-size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
+// The two-kernel path (qmm_frag.hip: a 16-bit scratch copy of the weights in fragment order, then a lean
+// GEMM) takes the shapes it wins on: at least eight rows of tiles to spread the copy over, tiles that fill
+// four fifths or more of their rounds of the CUs (it does not cut K), and no K cut planned for the fused kernel.
+bool prefer_frag_path(int64_t M, int64_t N, int64_t K, int gs, int bits) {
+  if (M < 2048 || !qmm_frag_shape_ok(M, N, K, bits) || use_mid_kernel(M, N, K)) return false;
+  const int cus = compute_units();
+  if (plan_tail(M, N, K, period_of(gs), cus).splits > 1) return false;
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const int64_t rounds = (tiles + cus - 1) / cus;
+  return tiles * 5 >= rounds * cus * 4;
+}
+
+size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
   if (K % BK) return 0;
   if (use_mid_kernel(M, N, K)) return qmm_mid_workspace_bytes(M, N, K, gs);
   return tail_plane_bytes(M, N, plan_tail(M, N, K, period_of(gs), compute_units()));
+}
+
+size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits) {
+  const size_t planes = qmm_min_workspace_bytes(M, N, K, gs);
+  if (!prefer_frag_path(M, N, K, gs, bits)) return planes;
+  const size_t copy = qmm_frag_workspace_bytes(N, K);
+  return copy > planes ? copy : planes;
 }
 
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
@@ -1148,6 +1167,10 @@ int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
   if (use_mid_kernel(M, N, K))
     return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
                           workspace_bytes, stream, low_rank, epi);
+  // the two-kernel path where it wins and the caller has brought room for the scratch copy
+  if (!low_rank.R && y_dtype == dtype && workspace && aligned16(workspace) &&
+      workspace_bytes >= qmm_frag_workspace_bytes(N, K) && prefer_frag_path(M, N, K, gs, bits))
+    return launch_qmm_frag(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
   if (epi.kind != kEpiNone)
     return launch_qmm_epilogue(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
                                workspace_bytes, stream, epi);

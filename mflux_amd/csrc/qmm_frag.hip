@@ -1,0 +1,487 @@
+// Large-M quantized GEMM in two kernels, for shapes whose 256x256 tiles fill the chip:
+//   1. dequant_frag_kernel expands the packed weights ONCE per call into 16-bit values
+//      (w_hat = round(fma(code, scale, bias)), the same single rounding as the fused
+//      kernels) and writes them in the order the matrix instructions consume them:
+//      blocks of 16 output rows x 64 k, 2 KiB each, laid out [half][lane][8 values], so
+//      that one 16-byte load per lane of a wavefront is a matrix fragment and one
+//      load instruction covers 1 KiB of contiguous memory;
+//   2. frag_gemm_kernel multiplies x with that scratch copy: 256x256x64 tiles, four
+//      wavefronts (one per SIMD, 256 rows x 64 columns each), v_mfma_f32_16x16x32
+//      with the weights as the A operand straight from global memory and x through
+//      LDS, persistent workgroups that prefetch across tile boundaries.
+// The fused kernel (qmm.hip) dequantises a weight once per 256 rows of x, M / 256
+// times per call, in the shadow of its matrix instructions; here that vector work is
+// gone from the matrix loop, which is what lets it use the 16-cycle instruction shape
+// (half the issue slots per matrix instruction).  The price is the scratch copy
+// (round_up(N, 16) * K * 2 bytes of workspace, HBM-bound to write) and a weight
+// operand four (W4) or two (W8) times larger for the GEMM to read.
+//
+// mx.quantized_matmul(x, w, scales, biases, transpose=True) of
+// src/mflux/models/common/weights/loading/weight_applier.py:43-103's quantized
+// linears, as qmm.hip.
+#include <type_traits>
+
+#include "common.h"
+#include "epilogue.h"
+
+namespace mfq {
+namespace {
+
+constexpr int BM = 256;
+constexpr int BN = 256;
+constexpr int BK = 64;
+constexpr int kThreads = 256;
+constexpr int kTileBytes = BM * BK * 2;          // one 16-bit x tile: 32 KiB
+constexpr int kStageStride = 144;                // bytes per staged output row: 64 16-bit columns + 16 bytes of padding
+constexpr int kStageBytes = 128 * kStageStride;  // one wavefront stages 128 rows of its 64 columns at a time
+constexpr int kBiasBytes = 64 * 4;               // per wavefront: the bias of its 64 columns as float32
+constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes + 4 * kBiasBytes;
+constexpr int kBlockBytes = 16 * BK * 2;         // one block of the scratch copy: 16 rows x 64 k
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// see qmm.hip: 128-bit LDS accesses are conflict free with the 16-byte column XORed with bits 1..3 of the row
+__device__ inline int swz(int row, int chunk) { return row * (BK * 2) + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+// see qmm.hip: XCD-contiguous runs of the tile sequence, bands of 4 tile rows, row index fastest
+__host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, int& m0, int& n0) {
+  const int n_tiles = tiles_m * tiles_n;
+  const int per_xcd = n_tiles / 8;
+  if (tile < per_xcd * 8) tile = (tile & 7) * per_xcd + (tile >> 3);
+  constexpr int kBandM = 4;
+  const int band_tiles = kBandM * tiles_n;
+  const int band = tile / band_tiles;
+  const int rest = tiles_m - band * kBandM;
+  const int band_rows = rest < kBandM ? rest : kBandM;
+  const int in_band = tile - band * band_tiles;
+  m0 = (band * kBandM + in_band % band_rows) * BM;
+  n0 = (in_band / band_rows) * BN;
+}
+
+// ---------------------------------------------------------------------------------------------
+// 1. the scratch copy.  One wavefront per block of 16 rows x 64 k and trip; lane (q, c16) = (lane / 16,
+// lane % 16) owns k [16 q, 16 q + 16) of row c16: 8 (W4) or 16 (W8) bytes of codes, one scale and one bias
+// (16 consecutive k lie in one group), two 16-byte stores, [half][lane].  Consecutive wavefronts take
+// consecutive blocks along K, so a row's codes are read in runs and every store instruction writes 1 KiB.
+template <typename T, int GS, int BITS>
+__global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __restrict__ wq,
+                                                           const uint16_t* __restrict__ scales,
+                                                           const uint16_t* __restrict__ biases,
+                                                           char* __restrict__ out, int N, int K, int n_blocks) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  using codes_t = std::conditional_t<BITS == 4, u32x2, u32x4>;  // 16 codes
+  constexpr int kPair = 2;  // blocks per wavefront and trip: neighbours along K (K / 64 is even), requested together
+  const int lane = threadIdx.x & (kWave - 1);
+  const int c16 = lane & 15, q = lane >> 4;
+  const int ks_per_row = K / BK;
+  const int waves = gridDim.x * 4;
+  for (int blk = (blockIdx.x * 4 + threadIdx.x / kWave) * kPair; blk < n_blocks; blk += waves * kPair) {
+    const int nb = blk / ks_per_row, ks = blk - nb * ks_per_row;
+    const int row = min(nb * 16 + c16, N - 1);  // rows past N repeat the last one; the GEMM never stores their columns
+    codes_t w[kPair];
+    float s[kPair], b[kPair];
+#pragma unroll
+    for (int u = 0; u < kPair; ++u) {
+      const int k0 = (ks + u) * BK + 16 * q;
+      w[u] = __builtin_nontemporal_load(reinterpret_cast<const codes_t*>(wq + ((int64_t)row * K + k0) * BITS / 32));
+      const int64_t g = (int64_t)row * (K / GS) + k0 / GS;
+      s[u] = T::to_f32(scales[g]), b[u] = T::to_f32(biases[g]);
+    }
+#pragma unroll
+    for (int u = 0; u < kPair; ++u) {
+      char* dst = out + (int64_t)(blk + u) * kBlockBytes + lane * 16;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        u32x4 o;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {  // values 2 p, 2 p + 1 of the half
+          float c0, c1;
+          if constexpr (BITS == 4) {
+            const uint32_t word = w[u][half] >> (8 * p);
+            c0 = (float)(word & 0xfu), c1 = (float)((word >> 4) & 0xfu);
+          } else {
+            const uint32_t word = w[u][2 * half + (p >> 1)] >> (16 * (p & 1));
+            c0 = (float)(word & 0xffu), c1 = (float)((word >> 8) & 0xffu);
+          }
+          o[p] = T::pack2(__builtin_fmaf(c0, s[u], b[u]), __builtin_fmaf(c1, s[u], b[u]));
+        }
+        // plain stores: the GEMM behind reads the copy back through the memory-side cache
+        *reinterpret_cast<u32x4*>(dst + 1024 * half) = o;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 2. the GEMM.
+//
+// The matrix instruction with its sum accumulated in place, as assembly: the compiler is free to give an
+// intrinsic's four result registers another place than its addend's, and with every one of the 256
+// accumulation registers holding part of the tile it then rotates accumulators through the vector
+// registers around every instruction.  Stated with the result tied to the addend, the instruction is
+// opaque to the compiler's hazard recognizer, so the kernel keeps every other instruction that touches
+// an accumulator (zeroing, the epilogue's reads) in other basic blocks than the matrix instructions and
+// separates them by settle() below; the build checks the generated code for that (_build.py).
+__device__ inline void mma16(bf16x8 a, bf16x8 b, f32x4& c) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ inline void mma16(f16x8 a, f16x8 b, f32x4& c) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+template <typename T, bool kEpi>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void frag_gemm_kernel(
+    const uint16_t* __restrict__ x, const char* __restrict__ wfrag, const uint16_t* __restrict__ bias,
+    void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, Epilogue epi) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  using vec8 = typename T::vec8;
+  const int n_items = tiles_m * tiles_n;
+  const int steps = K / BK;  // even, at least 4 (the launcher has checked)
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+  const int wn = wave * 64;
+  const int c16 = lane & 15;
+  const int q = lane >> 4;
+
+  // Per-lane byte offsets of the tile the PREFETCH cursor is in: the blocks of the wavefront's four column tiles
+  // (16 columns each; blocks past N repeat the last one) and the lane's eight x pieces (rows past M clamped).
+  uint32_t woff[4], xoff[8];
+  auto set_prefetch_tile = [&](int m0, int n0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t nb = (uint32_t)min((n0 + wn) / 16 + j, (N - 1) / 16);
+      woff[j] = nb * (uint32_t)steps * (uint32_t)kBlockBytes + (uint32_t)lane * 16u;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+  };
+  const char* xbytes = reinterpret_cast<const char*>(x);
+  const int wr_slot = swz(t >> 3, t & 7);
+  // x fragment of a pass: row c16 of a 16-row block (2048 bytes apart), 16-byte piece 2 q + pass, which holds
+  // k 16 q + 8 pass + [0, 8) of the step: the k a lane's weight fragment of that pass holds
+  int rd_slot[2];
+#pragma unroll
+  for (int half = 0; half < 2; ++half) rd_slot[half] = swz(c16, 2 * q + half);
+
+  u32x4 xa[8];        // the x tile on its way from global memory to LDS, one step ahead
+  vec8 wa[8], wb[8];  // weight fragments of the even / odd steps: [2 j + pass], column tile j
+  char* out_base = static_cast<char*>(y);
+  int out_stride = N;
+  const uint16_t* out_bias = bias;
+  f32x4 acc[16][4];   // [r][j][e]: row 16 r + c16, column 16 j + 4 q + e of the wavefront's 256 x 64 block
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+
+  auto load_w = [&](vec8 (&set)[8], int half, int step) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      set[2 * j + half] = *reinterpret_cast<const vec8*>(wfrag + (size_t)step * kBlockBytes + woff[j] + 1024 * half);
+  };
+
+  int m1 = 0, n1 = 0;  // the tile the prefetch cursor moves to in the middle of a tile's last-but-one step
+  // Step p = two passes of 64 matrix instructions (16 row blocks x 4 column tiles).  Behind them: every
+  // fourth slot the LDS read of the x fragment three row blocks ahead; in the first pass the request for
+  // the second-pass fragments of step p+1 into `other` (step p-1 has finished with them), in the second
+  // pass the request for the first-pass fragments of step p+2 into `now`; in the second pass also the LDS
+  // writes that publish the x tile of step p+1 and, behind each, the global load of that piece for step
+  // p+2.  s_h1 / s_h0: the steps (counted inside the cursor's tile) those requests are for; `sw`: the
+  // cursor enters the next tile between the passes.
+  auto do_step = [&](auto parity, bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
+      __attribute__((always_inline)) {
+    constexpr int kP = decltype(parity)::value;
+    const char* xs = lds + kP * kTileBytes;
+    char* xd = lds + (kP ^ 1) * kTileBytes;
+    vec8 xf[4];
+    auto read_frag = [&](int g) {  // g = 16 * pass + row block
+      xf[g & 3] = *reinterpret_cast<const vec8*>(xs + rd_slot[g >> 4] + 2048 * (g & 15));
+    };
+    read_frag(0);
+    read_frag(1);
+    read_frag(2);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      if (half == 1) {
+        if (sw) set_prefetch_tile(m1, n1);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int m = 4 * r + j;
+          const int g = 16 * half + r;
+          mma16(now[2 * j + half], xf[g & 3], acc[r][j]);
+          if (j == 0 && g + 3 < 32) read_frag(g + 3);
+          if (m == 1) {
+            if (half == 0) {
+              load_w(other, 1, s_h1);
+            } else {
+              load_w(now, 0, s_h0);
+            }
+          }
+          if (half == 1 && (m & 1) && m >= 17 && m < 33) {
+            const int i = (m - 17) >> 1;
+            *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * i) = xa[i];
+            xa[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)s_h0 * (BK * 2) + xoff[i]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  const std::integral_constant<int, 0> even_step{};
+  const std::integral_constant<int, 1> odd_step{};
+
+  // Fills the pipeline for the tile the cursor is in: x(0) into LDS buffer 0, x(1) into the registers, the
+  // fragments of step 0 and the first-pass fragments of step 1.
+  auto prime = [&]() {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i]);
+    load_w(wa, 0, 0);
+    load_w(wa, 1, 0);
+    load_w(wb, 0, 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + wr_slot + 4096 * i) = xa[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)(BK * 2) + xoff[i]);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // 16-bit output with N a multiple of 8: each wavefront transposes its 256 x 64 block through its
+  // private LDS region, 128 rows at a time (rows 144 bytes apart), so that every global store writes
+  // complete 128-byte row segments; the read-back applies the epilogues of epilogue.h.
+  auto store_tile_staged = [&](auto with_bias, int m0, int n0) {
+    constexpr bool kBias = decltype(with_bias)::value;
+    int lane_e = lane;  // opaque copy: keeps this per-tile address arithmetic out of the k loop's registers
+    asm volatile("" : "+v"(lane_e));
+    const int c16 = lane_e & 15;
+    const int q = lane_e >> 4;
+    const int lane = lane_e;
+    char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
+    uint16_t* yout = reinterpret_cast<uint16_t*>(out_base);
+    const float* bias_f = reinterpret_cast<const float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes);
+    if constexpr (kBias) {
+      *reinterpret_cast<float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes + lane * 4) =
+          T::to_f32(out_bias[min(n0 + wn + lane, N - 1)]);
+    }
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int cl = 16 * j + 4 * q;  // column inside the wavefront's 64
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (kBias) {
+          const float4 b4 = *reinterpret_cast<const float4*>(bias_f + cl);
+          bv[0] = b4.x, bv[1] = b4.y, bv[2] = b4.z, bv[3] = b4.w;
+        }
+#pragma unroll
+        for (int r8 = 0; r8 < 8; ++r8) {
+          const int r = 8 * pass + r8;
+          uint32_t pk[2];
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            pk[c] = T::pack2(acc[r][j][2 * c], acc[r][j][2 * c + 1]);
+            if constexpr (kBias)  // second rounding, as a separate add on the 16-bit result would do
+              pk[c] = T::pack2(lo_f32<T>(pk[c]) + bv[2 * c], hi_f32<T>(pk[c]) + bv[2 * c + 1]);
+          }
+          *reinterpret_cast<uint2*>(stage + (16 * r8 + c16) * kStageStride + cl * 2) = make_uint2(pk[0], pk[1]);
+          if (r8 & 1) __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      const int cg = n0 + wn + 8 * (lane & 7);
+      if constexpr (kEpi) {
+        if (epi.kind == kEpiSwiglu) {
+          const int cq = lane & 3;
+          const int co = (wn >> 1) + 8 * cq;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int rl = 16 * k + (lane >> 2);
+            const u32x4 g = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * cq);
+            const u32x4 u = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 64 + 16 * cq);
+            u32x4 v;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = epi_swiglu_pair<T>(g[c], u[c]);
+            const int row = m0 + 128 * pass + rl;
+            if (row < M && n0 + wn + 8 * cq < N)
+              *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + co) = v;
+          }
+          continue;
+        }
+        if (epi.kind == kEpiGateResidual) {
+          u32x4 gate8 = {0u, 0u, 0u, 0u};
+          if (cg < N) gate8 = *reinterpret_cast<const u32x4*>(epi.gate + cg);
+          const uint16_t* res = epi.residual + (int64_t)m0 * N + cg;
+#pragma unroll
+          for (int k4 = 0; k4 < 4; ++k4) {
+            u32x4 rv[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+              const int rl = 8 * (4 * k4 + kk) + (lane >> 3);
+              const int row = min(m0 + 128 * pass + rl, M - 1);
+              rv[kk] = cg < N ? *reinterpret_cast<const u32x4*>(res + (int64_t)(row - m0) * N) : gate8;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+              const int rl = 8 * (4 * k4 + kk) + (lane >> 3);
+              u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+#pragma unroll
+              for (int c = 0; c < 4; ++c) v[c] = epi_gate_residual_pair<T>(v[c], gate8[c], rv[kk][c]);
+              const int row = m0 + 128 * pass + rl;
+              if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
+            }
+          }
+          continue;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int rl = 8 * k + (lane >> 3);
+        u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
+        if constexpr (kEpi) {
+          if (epi.kind == kEpiGelu && cg >= epi.act_from) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[c] = epi_gelu_pair<T>(v[c]);
+          }
+        }
+        const int row = m0 + 128 * pass + rl;
+        if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
+        if (k & 1) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+
+  // Every accumulator in its accumulation register, and more wait states than any matrix instruction needs
+  // between the instructions in front and behind.
+  auto settle = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 16; r += 4)
+      asm volatile("s_nop 15\n\ts_nop 15"
+                   : "+a"(acc[r][0]), "+a"(acc[r][1]), "+a"(acc[r][2]), "+a"(acc[r][3]), "+a"(acc[r + 1][0]),
+                     "+a"(acc[r + 1][1]), "+a"(acc[r + 1][2]), "+a"(acc[r + 1][3]), "+a"(acc[r + 2][0]),
+                     "+a"(acc[r + 2][1]), "+a"(acc[r + 2][2]), "+a"(acc[r + 2][3]), "+a"(acc[r + 3][0]),
+                     "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]), "+a"(acc[r + 3][3]));
+  };
+
+  bool primed = false;
+  for (int seq = blockIdx.x; seq < n_items; seq += gridDim.x) {
+    int m0, n0;
+    tile_origin(seq, tiles_m, tiles_n, m0, n0);
+    out_base = static_cast<char*>(y) + ((size_t)m0 * N + n0) * 2;
+    out_stride = N;
+    if constexpr (kEpi) {
+      if (epi.kind == kEpiSwiglu) {
+        out_base = static_cast<char*>(y) + ((size_t)m0 * (N / 2) + n0 / 2) * 2;
+        out_stride = N / 2;
+      }
+    }
+    if (!primed) {
+      set_prefetch_tile(m0, n0);
+      prime();
+    }
+    const bool has_next = seq + (int)gridDim.x < n_items;
+    m1 = m0, n1 = n0;
+    if (has_next) tile_origin(seq + gridDim.x, tiles_m, tiles_n, m1, n1);
+    const int s_next = has_next ? 0 : steps - 2;  // without a next tile: the last pair again (loaded, not used)
+    settle();
+    // ONE body for every pair of steps, the tile's last included: the accumulators pass through a single
+    // copy of the matrix instructions, so the compiler has no place to move them between register files
+    for (int p = 0; p < steps; p += 2) {
+      const bool last = p == steps - 2;
+      do_step(even_step, last, wa, wb, p + 1, last ? s_next : p + 2);
+      do_step(odd_step, false, wb, wa, last ? s_next : p + 2, last ? s_next + 1 : p + 3);
+    }
+    settle();
+    primed = has_next;
+    if (out_bias) {
+      store_tile_staged(std::true_type{}, m0, n0);
+    } else {
+      store_tile_staged(std::false_type{}, m0, n0);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  }
+}
+
+template <typename T, int GS>
+int launch_dequant_bits(const uint32_t* wq, const void* scales, const void* biases, int bits, void* out, int64_t N,
+                        int64_t K, hipStream_t stream) {
+  const int64_t n_blocks = ((N + 15) / 16) * (K / BK);
+  const int64_t wanted = (n_blocks / 2 + 3) / 4;  // a wavefront takes two blocks per trip
+  const int cap = compute_units() * 16;
+  const dim3 grid((unsigned)(wanted < cap ? wanted : cap));
+  if (bits == 4) {
+    hipLaunchKernelGGL((dequant_frag_kernel<T, GS, 4>), grid, dim3(256), 0, stream, wq, (const uint16_t*)scales,
+                       (const uint16_t*)biases, (char*)out, (int)N, (int)K, (int)n_blocks);
+  } else {
+    hipLaunchKernelGGL((dequant_frag_kernel<T, GS, 8>), grid, dim3(256), 0, stream, wq, (const uint16_t*)scales,
+                       (const uint16_t*)biases, (char*)out, (int)N, (int)K, (int)n_blocks);
+  }
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T>
+int launch_dequant(const uint32_t* wq, const void* scales, const void* biases, int gs, int bits, void* out, int64_t N,
+                   int64_t K, hipStream_t stream) {
+  if (gs == 32) return launch_dequant_bits<T, 32>(wq, scales, biases, bits, out, N, K, stream);
+  if (gs == 64) return launch_dequant_bits<T, 64>(wq, scales, biases, bits, out, N, K, stream);
+  return launch_dequant_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
+}
+
+template <typename T, bool kEpi>
+int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const void* bias, int64_t N, void* y,
+                hipStream_t stream, Epilogue epi) {
+  auto kernel = frag_gemm_kernel<T, kEpi>;
+  static PerDeviceInt configured;
+  if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
+  const int tiles_m = (int)((M + BM - 1) / BM);
+  const int tiles_n = (int)((N + BN - 1) / BN);
+  const int n_items = tiles_m * tiles_n;
+  const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x,
+                     (const char*)wfrag, (const uint16_t*)bias, y, (int)M, (int)N, (int)K, tiles_m, tiles_n, epi);
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+
+template <typename T>
+int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
+                 const void* bias, int64_t N, int gs, int bits, void* y, void* workspace, hipStream_t stream,
+                 Epilogue epi) {
+  if (int rc = launch_dequant<T>(wq, scales, biases, gs, bits, workspace, N, K, stream)) return rc;
+  if (epi.kind != kEpiNone) return launch_gemm<T, true>(x, M, K, workspace, bias, N, y, stream, epi);
+  return launch_gemm<T, false>(x, M, K, workspace, bias, N, y, stream, epi);
+}
+
+}  // namespace
+
+bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits) {
+  // whole pairs of k steps and at least two of them; whole 16-byte pieces of y; 32-bit byte offsets into x
+  // and into the scratch copy
+  return (bits == 4 || bits == 8) && K % (2 * BK) == 0 && K >= 4 * BK && N % 8 == 0 && M * K < ((int64_t)1 << 31) &&
+         ((N + 15) / 16) * 16 * K < ((int64_t)1 << 31);
+}
+
+size_t qmm_frag_workspace_bytes(int64_t N, int64_t K) { return (size_t)(((N + 15) / 16) * 16 * K * 2); }
+
+int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
+                    hipStream_t stream, Epilogue epi) {
+  if (!qmm_frag_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+  if (dtype == MFQ_BF16)
+    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
+  if (dtype == MFQ_F16)
+    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
+  return MFQ_EDTYPE;
+}
+
+}  // namespace mfq

@@ -1,0 +1,151 @@
+"""GPU parity of the two-kernel large-M path (csrc/qmm_frag.hip): the scratch
+copy of the weights is bit-identical to the oracle's dequantisation, laid out in
+fragment order, and the product meets the matmul tolerance (1e-2 of the row's
+largest reference magnitude) against the float64 oracle; the fused kernel, which
+the same call falls back to without a workspace, agrees within the same bound.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import seeded
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _operands(o, cfg, M, K, N, bits, gs, dt, with_bias):
+    def to_bits(a):
+        return o._from_f32(a, dt)
+
+    x = to_bits(seeded(cfg, 0, (M, K), 1.0))
+    w = to_bits(seeded(cfg, 1, (N, K), 0.02))
+    bias = to_bits(seeded(cfg, 2, (N,), 0.02)) if with_bias else None
+    wq, s, b = o.c_quantize(w, dt, gs, bits)
+    return x, wq, s, b, bias
+
+
+def _to_f64(o, bits16, dt):
+    return o._to_f32(bits16, dt).astype(np.float64)
+
+
+def _call(lib, name, code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y, ws, ws_bytes):
+    return getattr(lib, name)(xd.data_ptr(), code, M, K, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), code,
+                              None if biasd is None else biasd.data_ptr(), N, gs, bits, y.data_ptr(), code,
+                              None if ws is None else ws.data_ptr(), ws_bytes,
+                              torch.cuda.current_stream().cuda_stream)
+
+
+# 17 x 13 tiles = 221 of 256 CUs: the shape class the path takes; M and N ragged (N % 16 == 8)
+@pytest.mark.parametrize("bits,gs,dtype,with_bias", [
+    (4, 64, "bf16", True), (8, 64, "bf16", False), (4, 32, "bf16", False), (8, 128, "bf16", True),
+    (4, 128, "f16", True), (8, 32, "f16", False)])
+def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_bias):
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    M, K, N = 4100, 512, 3208
+    need = lib.mfq_qmm_t_workspace_bytes(M, K, N, gs, bits)
+    n16 = (N + 15) // 16 * 16
+    assert need == n16 * K * 2, "the shape must take the two-kernel path"
+    x, wq, s, b, bias = _operands(o, 90 + bits + gs, M, K, N, bits, gs, dt, with_bias)
+    xd, wd, sd, bd = to_dev(x, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt)
+    biasd = None if bias is None else to_dev(bias, dt)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    y = torch.empty(M, N, dtype=xd.dtype, device="cuda")
+    assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y, ws, need) == 0
+    torch.cuda.synchronize()
+
+    # the scratch copy: blocks of 16 rows x 64 k as [half][q][c16][8], value (q, half, e) = k 16 q + 8 half + e
+    copy = ws.view(torch.int16).view(n16 // 16, K // 64, 2, 4, 16, 8).permute(0, 4, 1, 3, 2, 5).reshape(n16, K)
+    got = copy.cpu().numpy().view(np.uint16)
+    w_hat = o.dequantize_exact(wq, s, b, dt, gs, bits).astype(np.float32)  # float32 fma of exact operands
+    want = o._from_f32(w_hat, dt)
+    assert np.array_equal(got[:N], want)
+    assert np.array_equal(got[N:], np.broadcast_to(want[N - 1], (n16 - N, K)))  # rows past N repeat the last one
+
+    ref = o.quantized_matmul_f64(_to_f64(o, x, dt), wq, s, b, dt, gs, bits,
+                                 bias_f64=None if bias is None else _to_f64(o, bias, dt))
+    row_inf = np.abs(ref).max(axis=-1, keepdims=True)
+    err = np.abs(y.double().cpu().numpy() - ref) / row_inf
+    assert err.max() <= TOL, err.max()
+
+    # without a workspace the fused kernel takes the call: same bound, and close to the two-kernel result
+    y_fused = torch.empty_like(y)
+    assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y_fused, None, 0) == 0
+    torch.cuda.synchronize()
+    err_fused = np.abs(y_fused.double().cpu().numpy() - ref) / row_inf
+    assert err_fused.max() <= TOL, err_fused.max()
+    assert not torch.equal(y_fused, torch.zeros_like(y_fused))
+
+
+def test_two_kernel_path_is_chosen_for_full_rounds_only():
+    """The workspace the library asks for tells which path a shape takes: the scratch
+    copy for shapes whose tiles fill their rounds, the K split's planes (or
+    nothing) for the others."""
+    from mflux_amd import _lib
+
+    lib = _lib.load()
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("tile counts below are for 256 CUs")
+    q = lib.mfq_qmm_t_workspace_bytes
+    assert q(4608, 3072, 21504, 64, 4) == 21504 * 3072 * 2      # FLUX single block, linear1
+    assert q(4608, 15360, 3072, 64, 4) == 3072 * 15360 * 2      # linear2: 216 tiles
+    assert q(4352, 3840, 10240, 64, 8) == 10240 * 3840 * 2      # Z-Image
+    assert q(4096, 3072, 3072, 64, 4) == 0                      # 192 tiles: three quarters of a round, fused kernel
+    assert q(1024, 3072, 21504, 64, 4) < 21504 * 3072 * 2       # four rows of tiles: the copy would not pay
+    planes = q(6889, 3072, 3072, 64, 4)                         # one round + 68 tiles: the fused kernel's K split
+    assert 0 < planes and planes % (256 * 256 * 4) == 0
+    assert q(4608, 3072, 21504, 64, 5) != 21504 * 3072 * 2      # odd bit widths have their own kernel
+
+
+def test_two_kernel_path_epilogues_and_graph_replay(oracle):
+    """GELU from a column on, gate * y + residual and SwiGLU through the two-kernel
+    path against the composed reference, and a captured call replayed bit for bit."""
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    M, K, N, bits = 4100, 512, 3200, 4
+    x, wq, s, b, bias = _operands(o, 97, M, K, N, bits, 64, o.BF16, True)
+    xd, wd, sd, bd, biasd = to_dev(x, o.BF16), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16), to_dev(bias, o.BF16)
+    gate = to_dev(o.f32_to_bf16_bits(seeded(97, 3, (N,), 1.0)), o.BF16)
+    res = to_dev(o.f32_to_bf16_bits(seeded(97, 4, (M, N), 1.0)), o.BF16)
+    plain = mflux_amd.quantized_matmul(xd, wd, sd, bd, bits=bits, bias=biasd)
+
+    def close(got, want, extra_roundings):
+        bound = TOL + extra_roundings * 2.0 ** -8
+        scale = want.double().abs().amax(dim=-1, keepdim=True).clamp_min(1e-30)
+        err = ((got.double() - want.double()).abs() / scale).max().item()
+        assert err <= bound, err
+
+    y = mflux_amd.quantized_matmul_epilogue(xd, wd, sd, bd, epilogue="gelu", bits=bits, bias=biasd, act_from=1600)
+    want = torch.cat([plain[:, :1600], mflux_amd.gelu_approx(plain[:, 1600:])], dim=-1)
+    close(y, want, 1)
+    y = mflux_amd.quantized_matmul_epilogue(xd, wd, sd, bd, epilogue="gate_residual", bits=bits, bias=biasd, gate=gate,
+                                            residual=res)
+    close(y, res + gate * plain, 2)
+    y = mflux_amd.quantized_matmul_epilogue(xd, wd, sd, bd, epilogue="swiglu", bits=bits, bias=biasd)
+    close(y, mflux_amd.core.swiglu_unstack(plain), 3)
+
+    # graph capture: the workspace comes from torch's allocator inside the capture; every replay equals the eager result
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        mflux_amd.quantized_matmul(xd, wd, sd, bd, bits=bits, bias=biasd)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_g = mflux_amd.quantized_matmul(xd, wd, sd, bd, bits=bits, bias=biasd)
+    for _ in range(3):
+        y_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, plain)
+        mflux_amd.quantized_matmul(xd, wd, sd, bd, bits=bits)  # eager work between the replays
+        torch.cuda.synchronize()
