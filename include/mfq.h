@@ -212,11 +212,20 @@ int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* 
  * cut into ranges that run on different compute units, each range accumulates
  * into its own float32 plane of the workspace, and a second kernel adds the
  * planes, rounds and applies the bias (same two roundings as the fused
- * epilogue).  mfq_qmm_t_workspace_bytes() returns the size this shape would
- * use on the current device (0: K is not split, pass NULL).  A NULL or smaller
- * workspace is not an error: the call then runs as mfq_qmm_t does.  The
- * workspace must be 16-byte aligned; its contents before and after the call
- * are undefined; calls sharing one workspace must be ordered on one stream.
+ * epilogue).  The opposite shapes -- 4 or 8 bits, 16-bit y, at least 2048
+ * activation rows and tiles that fill four fifths or more of their rounds of
+ * the compute units, e.g. the single-stream linears of FLUX.1 at M = 4608 --
+ * use the workspace for a 16-bit copy of the dequantised weights
+ * (round_up(N, 16) * K * 2 bytes, written once per call in the order the matrix
+ * instructions consume it) and multiply with a kernel that has no
+ * dequantisation in its loop; the copy's values are the ones the fused kernels
+ * use (one rounding of fma(code, scale, bias)), the float32 sums run in another
+ * order.  mfq_qmm_t_workspace_bytes() returns the size this shape would use on
+ * the current device (0: neither applies, pass NULL).  A NULL or smaller
+ * workspace is not an error: the call then runs as mfq_qmm_t does (the fused
+ * kernel, K not split).  The workspace must be 16-byte aligned; its contents
+ * before and after the call are undefined; calls sharing one workspace must be
+ * ordered on one stream.
  */
 size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits);
 int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
@@ -232,7 +241,9 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
  * GPU the library runs on holds its own copy until the process ends), so the
  * call allocates nothing and takes no workspace: same arguments as mfq_qmm_t,
  * same kernels and bit-identical results as mfq_qmm_t_ws with a workspace of
- * mfq_qmm_t_workspace_bytes().  A shape whose split needs more than the
+ * mfq_qmm_t_workspace_bytes() -- except that a copy of the dequantised weights
+ * that does not fit the buffer is done without (the fused kernel then runs:
+ * same tolerance, other bits).  A shape whose split needs more than the
  * buffer holds is refused with MFQ_ESCRATCH and nothing is launched (on a
  * 256-CU device: the last, short round of 256 x 256 tiles cut into more than
  * 128 planes, e.g. M = 6889 against 3072 -> 3072; use mfq_qmm_t_ws or

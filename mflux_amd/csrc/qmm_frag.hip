@@ -7,8 +7,9 @@
 //      load instruction covers 1 KiB of contiguous memory;
 //   2. frag_gemm_kernel multiplies x with that scratch copy: 256x256x64 tiles, four
 //      wavefronts (one per SIMD, 256 rows x 64 columns each), v_mfma_f32_16x16x32
-//      with the weights as the A operand straight from global memory and x through
-//      LDS, persistent workgroups that prefetch across tile boundaries.
+//      with the weights as the A operand straight from global memory into registers
+//      and x from global memory straight into LDS (three tiles, no registers in
+//      between), persistent workgroups that prefetch across tile boundaries.
 // The fused kernel (qmm.hip) dequantises a weight once per 256 rows of x, M / 256
 // times per call, in the shadow of its matrix instructions; here that vector work is
 // gone from the matrix loop, which is what lets it use the 16-cycle instruction shape
@@ -33,9 +34,11 @@ constexpr int BK = 64;
 constexpr int kThreads = 256;
 constexpr int kTileBytes = BM * BK * 2;          // one 16-bit x tile: 32 KiB
 constexpr int kStageStride = 144;                // bytes per staged output row: 64 16-bit columns + 16 bytes of padding
-constexpr int kStageBytes = 128 * kStageStride;  // one wavefront stages 128 rows of its 64 columns at a time
+constexpr int kStageRows = 64;                   // one wavefront stages 64 rows of its 64 columns at a time
+constexpr int kStageBytes = kStageRows * kStageStride;
 constexpr int kBiasBytes = 64 * 4;               // per wavefront: the bias of its 64 columns as float32
-constexpr int kLdsBytes = 2 * kTileBytes + 4 * kStageBytes + 4 * kBiasBytes;
+constexpr int kXBuffers = 3;                     // x tiles in LDS: in use, next, being filled
+constexpr int kLdsBytes = kXBuffers * kTileBytes + 4 * kStageBytes + 4 * kBiasBytes;
 constexpr int kBlockBytes = 16 * BK * 2;         // one block of the scratch copy: 16 rows x 64 k
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -63,14 +66,14 @@ __host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, 
 // lane % 16) owns k [16 q, 16 q + 16) of row c16: 8 (W4) or 16 (W8) bytes of codes, one scale and one bias
 // (16 consecutive k lie in one group), two 16-byte stores, [half][lane].  Consecutive wavefronts take
 // consecutive blocks along K, so a row's codes are read in runs and every store instruction writes 1 KiB.
-template <typename T, int GS, int BITS>
+// kPair: blocks per wavefront and trip, neighbours along K (K / 64 is a multiple of it), requested together.
+template <typename T, int GS, int BITS, int kPair>
 __global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __restrict__ wq,
                                                            const uint16_t* __restrict__ scales,
                                                            const uint16_t* __restrict__ biases,
                                                            char* __restrict__ out, int N, int K, int n_blocks) {
   typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
   using codes_t = std::conditional_t<BITS == 4, u32x2, u32x4>;  // 16 codes
-  constexpr int kPair = 2;  // blocks per wavefront and trip: neighbours along K (K / 64 is even), requested together
   const int lane = threadIdx.x & (kWave - 1);
   const int c16 = lane & 15, q = lane >> 4;
   const int ks_per_row = K / BK;
@@ -153,19 +156,30 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       const uint32_t nb = (uint32_t)min((n0 + wn) / 16 + j, (N - 1) / 16);
       woff[j] = nb * (uint32_t)steps * (uint32_t)kBlockBytes + (uint32_t)lane * 16u;
     }
+    // lane l of a direct load lands in LDS at 16 l past the load's base: row l / 8 of the wavefront's eight,
+    // 16-byte slot l % 8, which in the swizzled tile holds the row's piece (l % 8) ^ ((row / 2) % 8)
+    const uint32_t piece = (uint32_t)((t & 7) ^ (((t >> 3) >> 1) & 7));  // 32 i rows further on: the same
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * (t & 7)) * 2u;
+      xoff[i] = ((uint32_t)min(m0 + (t >> 3) + 32 * i, M - 1) * (uint32_t)K + 8u * piece) * 2u;
   };
   const char* xbytes = reinterpret_cast<const char*>(x);
-  const int wr_slot = swz(t >> 3, t & 7);
+  // 16 bytes per lane from global memory straight into LDS, 1 KiB per instruction (eight rows of the tile):
+  // no registers, no LDS write instructions.  The compiler does not see these loads; it counts only the
+  // weight loads, so its own waits can only be stricter than it thinks, and the waits for the tiles
+  // themselves are stated below by count.
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  auto dma16 = [&](const char* sbase, uint32_t voff, uint32_t lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory", "m0");
+  };
+  int x_cur = 0, x_next = kTileBytes, x_fill = 2 * kTileBytes;  // LDS offsets of the three x tiles
   // x fragment of a pass: row c16 of a 16-row block (2048 bytes apart), 16-byte piece 2 q + pass, which holds
   // k 16 q + 8 pass + [0, 8) of the step: the k a lane's weight fragment of that pass holds
   int rd_slot[2];
 #pragma unroll
   for (int half = 0; half < 2; ++half) rd_slot[half] = swz(c16, 2 * q + half);
 
-  u32x4 xa[8];        // the x tile on its way from global memory to LDS, one step ahead
   vec8 wa[8], wb[8];  // weight fragments of the even / odd steps: [2 j + pass], column tile j
   char* out_base = static_cast<char*>(y);
   int out_stride = N;
@@ -188,15 +202,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // Step p = two passes of 64 matrix instructions (16 row blocks x 4 column tiles).  Behind them: every
   // fourth slot the LDS read of the x fragment three row blocks ahead; in the first pass the request for
   // the second-pass fragments of step p+1 into `other` (step p-1 has finished with them), in the second
-  // pass the request for the first-pass fragments of step p+2 into `now`; in the second pass also the LDS
-  // writes that publish the x tile of step p+1 and, behind each, the global load of that piece for step
-  // p+2.  s_h1 / s_h0: the steps (counted inside the cursor's tile) those requests are for; `sw`: the
-  // cursor enters the next tile between the passes.
-  auto do_step = [&](auto parity, bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
+  // pass the request for the first-pass fragments of step p+2 into `now` and the eight direct loads of
+  // the x tile of step p+2 into the LDS tile that step p-1 read -- one load every eighth (weights) or
+  // seventh (x) slot rather than in a burst, which measured 1 % faster.  s_h1 / s_h0: the steps (counted inside
+  // the cursor's tile) those requests are for; `sw`: the cursor enters the next tile between the passes.
+  auto do_step = [&](bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
       __attribute__((always_inline)) {
-    constexpr int kP = decltype(parity)::value;
-    const char* xs = lds + kP * kTileBytes;
-    char* xd = lds + (kP ^ 1) * kTileBytes;
+    const char* xs = lds + x_cur;
+    const uint32_t fill = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)x_fill + (uint32_t)wave * 1024u);
     vec8 xf[4];
     auto read_frag = [&](int g) {  // g = 16 * pass + row block
       xf[g & 3] = *reinterpret_cast<const vec8*>(xs + rd_slot[g >> 4] + 2048 * (g & 15));
@@ -217,45 +230,53 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           const int g = 16 * half + r;
           mma16(now[2 * j + half], xf[g & 3], acc[r][j]);
           if (j == 0 && g + 3 < 32) read_frag(g + 3);
-          if (m == 1) {
+          if ((m & 7) == 2 && m < 32) {
+            const int j1 = m >> 3;
             if (half == 0) {
-              load_w(other, 1, s_h1);
+              other[2 * j1 + 1] = *reinterpret_cast<const vec8*>(wfrag + (size_t)s_h1 * kBlockBytes + woff[j1] + 1024);
             } else {
-              load_w(now, 0, s_h0);
+              now[2 * j1] = *reinterpret_cast<const vec8*>(wfrag + (size_t)s_h0 * kBlockBytes + woff[j1]);
             }
           }
-          if (half == 1 && (m & 1) && m >= 17 && m < 33) {
-            const int i = (m - 17) >> 1;
-            *reinterpret_cast<u32x4*>(xd + wr_slot + 4096 * i) = xa[i];
-            xa[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)s_h0 * (BK * 2) + xoff[i]);
+          if (half == 1 && m >= 6 && (m - 6) % 7 == 0 && m < 6 + 56) {
+            const int i = (m - 6) / 7;
+            dma16(xbytes + (size_t)s_h0 * (BK * 2), xoff[i], fill + 4096u * i);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
     }
+    // The x tile of the next step, requested during the previous step, must have landed in every wavefront's
+    // part before anyone reads it: younger than those requests are the 8 weight loads and the 8 direct loads
+    // of this step (stores of a tile's epilogue in between only make the count stricter).
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
+    const int done = x_cur;
+    x_cur = x_next;
+    x_next = x_fill;
+    x_fill = done;
   };
-  const std::integral_constant<int, 0> even_step{};
-  const std::integral_constant<int, 1> odd_step{};
 
-  // Fills the pipeline for the tile the cursor is in: x(0) into LDS buffer 0, x(1) into the registers, the
+  // Fills the pipeline for the tile the cursor is in: x(0) and x(1) into LDS, the
   // fragments of step 0 and the first-pass fragments of step 1.
   auto prime = [&]() {
+    const uint32_t w1k = lds_base + (uint32_t)wave * 1024u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(xbytes + xoff[i]);
+    for (int i = 0; i < 8; ++i)
+      dma16(xbytes, xoff[i], __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_cur) + 4096u * i);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      dma16(xbytes + (size_t)(BK * 2), xoff[i], __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_next) + 4096u * i);
     load_w(wa, 0, 0);
     load_w(wa, 1, 0);
     load_w(wb, 0, 1);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(lds + wr_slot + 4096 * i) = xa[i];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) xa[i] = *reinterpret_cast<const u32x4*>(xbytes + (size_t)(BK * 2) + xoff[i]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both x tiles have landed (the fragments too)
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
   };
 
   // 16-bit output with N a multiple of 8: each wavefront transposes its 256 x 64 block through its
-  // private LDS region, 128 rows at a time (rows 144 bytes apart), so that every global store writes
+  // private LDS region, 64 rows at a time (rows 144 bytes apart), so that every global store writes
   // complete 128-byte row segments; the read-back applies the epilogues of epilogue.h.
   auto store_tile_staged = [&](auto with_bias, int m0, int n0) {
     constexpr bool kBias = decltype(with_bias)::value;
@@ -264,15 +285,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int c16 = lane_e & 15;
     const int q = lane_e >> 4;
     const int lane = lane_e;
-    char* stage = lds + 2 * kTileBytes + wave * kStageBytes;
+    char* stage = lds + kXBuffers * kTileBytes + wave * kStageBytes;
     uint16_t* yout = reinterpret_cast<uint16_t*>(out_base);
-    const float* bias_f = reinterpret_cast<const float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes);
+    const float* bias_f = reinterpret_cast<const float*>(lds + kXBuffers * kTileBytes + 4 * kStageBytes + wave * kBiasBytes);
     if constexpr (kBias) {
-      *reinterpret_cast<float*>(lds + 2 * kTileBytes + 4 * kStageBytes + wave * kBiasBytes + lane * 4) =
+      *reinterpret_cast<float*>(lds + kXBuffers * kTileBytes + 4 * kStageBytes + wave * kBiasBytes + lane * 4) =
           T::to_f32(out_bias[min(n0 + wn + lane, N - 1)]);
     }
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < 256 / kStageRows; ++pass) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int cl = 16 * j + 4 * q;  // column inside the wavefront's 64
@@ -282,8 +303,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           bv[0] = b4.x, bv[1] = b4.y, bv[2] = b4.z, bv[3] = b4.w;
         }
 #pragma unroll
-        for (int r8 = 0; r8 < 8; ++r8) {
-          const int r = 8 * pass + r8;
+        for (int r8 = 0; r8 < kStageRows / 16; ++r8) {
+          const int r = kStageRows / 16 * pass + r8;
           uint32_t pk[2];
 #pragma unroll
           for (int c = 0; c < 2; ++c) {
@@ -301,14 +322,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           const int cq = lane & 3;
           const int co = (wn >> 1) + 8 * cq;
 #pragma unroll
-          for (int k = 0; k < 8; ++k) {
+          for (int k = 0; k < kStageRows / 16; ++k) {
             const int rl = 16 * k + (lane >> 2);
             const u32x4 g = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * cq);
             const u32x4 u = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 64 + 16 * cq);
             u32x4 v;
 #pragma unroll
             for (int c = 0; c < 4; ++c) v[c] = epi_swiglu_pair<T>(g[c], u[c]);
-            const int row = m0 + 128 * pass + rl;
+            const int row = m0 + kStageRows * pass + rl;
             if (row < M && n0 + wn + 8 * cq < N)
               *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + co) = v;
           }
@@ -319,12 +340,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           if (cg < N) gate8 = *reinterpret_cast<const u32x4*>(epi.gate + cg);
           const uint16_t* res = epi.residual + (int64_t)m0 * N + cg;
 #pragma unroll
-          for (int k4 = 0; k4 < 4; ++k4) {
+          for (int k4 = 0; k4 < kStageRows / 32; ++k4) {
             u32x4 rv[4];
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
               const int rl = 8 * (4 * k4 + kk) + (lane >> 3);
-              const int row = min(m0 + 128 * pass + rl, M - 1);
+              const int row = min(m0 + kStageRows * pass + rl, M - 1);
               rv[kk] = cg < N ? *reinterpret_cast<const u32x4*>(res + (int64_t)(row - m0) * N) : gate8;
             }
 #pragma unroll
@@ -333,7 +354,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
               u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
 #pragma unroll
               for (int c = 0; c < 4; ++c) v[c] = epi_gate_residual_pair<T>(v[c], gate8[c], rv[kk][c]);
-              const int row = m0 + 128 * pass + rl;
+              const int row = m0 + kStageRows * pass + rl;
               if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
             }
           }
@@ -341,7 +362,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
       }
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
+      for (int k = 0; k < kStageRows / 8; ++k) {
         const int rl = 8 * k + (lane >> 3);
         u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * (lane & 7));
         if constexpr (kEpi) {
@@ -350,7 +371,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (int c = 0; c < 4; ++c) v[c] = epi_gelu_pair<T>(v[c]);
           }
         }
-        const int row = m0 + 128 * pass + rl;
+        const int row = m0 + kStageRows * pass + rl;
         if (row < M && cg < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (cg - n0)) = v;
         if (k & 1) __builtin_amdgcn_sched_barrier(0);
       }
@@ -394,8 +415,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     // copy of the matrix instructions, so the compiler has no place to move them between register files
     for (int p = 0; p < steps; p += 2) {
       const bool last = p == steps - 2;
-      do_step(even_step, last, wa, wb, p + 1, last ? s_next : p + 2);
-      do_step(odd_step, false, wb, wa, last ? s_next : p + 2, last ? s_next + 1 : p + 3);
+      do_step(last, wa, wb, p + 1, last ? s_next : p + 2);
+      do_step(false, wb, wa, last ? s_next : p + 2, last ? s_next + 1 : p + 3);
     }
     settle();
     primed = has_next;
@@ -417,15 +438,18 @@ template <typename T, int GS>
 int launch_dequant_bits(const uint32_t* wq, const void* scales, const void* biases, int bits, void* out, int64_t N,
                         int64_t K, hipStream_t stream) {
   const int64_t n_blocks = ((N + 15) / 16) * (K / BK);
-  const int64_t wanted = (n_blocks / 2 + 3) / 4;  // a wavefront takes two blocks per trip
+  const bool four = (K / BK) % 4 == 0;
+  const int64_t wanted = (n_blocks / (four ? 4 : 2) + 3) / 4;
   const int cap = compute_units() * 16;
   const dim3 grid((unsigned)(wanted < cap ? wanted : cap));
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, wq, (const uint16_t*)scales, (const uint16_t*)biases,
+                       (char*)out, (int)N, (int)K, (int)n_blocks);
+  };
   if (bits == 4) {
-    hipLaunchKernelGGL((dequant_frag_kernel<T, GS, 4>), grid, dim3(256), 0, stream, wq, (const uint16_t*)scales,
-                       (const uint16_t*)biases, (char*)out, (int)N, (int)K, (int)n_blocks);
+    if (four) launch(dequant_frag_kernel<T, GS, 4, 4>); else launch(dequant_frag_kernel<T, GS, 4, 2>);
   } else {
-    hipLaunchKernelGGL((dequant_frag_kernel<T, GS, 8>), grid, dim3(256), 0, stream, wq, (const uint16_t*)scales,
-                       (const uint16_t*)biases, (char*)out, (int)N, (int)K, (int)n_blocks);
+    if (four) launch(dequant_frag_kernel<T, GS, 8, 4>); else launch(dequant_frag_kernel<T, GS, 8, 2>);
   }
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
