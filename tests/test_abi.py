@@ -192,3 +192,15 @@ def test_abi_validation_clean_under_host_sanitizers():
     from mflux_amd import _build
 
     assert "every refusal clean" in _build.sanitize_abi()
+
+
+def test_no_accumulator_moves_next_to_assembly_matrix_instructions():
+    """The two-kernel GEMM states its matrix instruction as assembly (result tied
+    to the addend), which hides it from the compiler's hazard recognizer; the
+    build therefore refuses generated code in which a basic block holds both such
+    an instruction and a move of an accumulator between register files.  The
+    check runs here on a fresh compile: four kernels (two types x with / without
+    epilogue), all clean."""
+    from mflux_amd import _build
+
+    assert _build.check_accumulator_moves("qmm_frag.hip") == 4
