@@ -350,14 +350,18 @@ int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void*
 // preferred) and what the call cannot do without (the planes only)
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits);
 size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
-// the two-kernel path (qmm_frag.hip): dequantize once into a 16-bit copy in fragment order (workspace:
-// qmm_frag_workspace_bytes, 16-byte aligned), then a GEMM on 16x16x32 matrix instructions; 4 and 8 bits,
-// 16-bit y of x's type, epilogues as launch_qmm_epilogue
+// the two-kernel path (qmm_frag.hip): dequantize once into a 16-bit copy in fragment order, then a GEMM on
+// 16x16x32 matrix instructions; 4 and 8 bits, 16-bit y of x's type, epilogues as launch_qmm_epilogue.
+// workspace (16-byte aligned): qmm_frag_copy_bytes(N, K) for the copy and, behind it, the float32 planes of a
+// K cut (n_whole whole tiles, the others in `splits` ranges of whole pairs of k steps; splits == 1: no cut)
 bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits);
-size_t qmm_frag_workspace_bytes(int64_t N, int64_t K);
+size_t qmm_frag_copy_bytes(int64_t N, int64_t K);
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
-                    hipStream_t stream, Epilogue epi);
+                    int n_whole, int splits, hipStream_t stream, Epilogue epi);
+// y tiles = sums of the planes of a K cut (+ bias, epilogue): the second kernel of qmm.hip's and qmm_frag.hip's cut
+int launch_tail_reduce(int dtype, const float* planes, int n_whole, int splits, int tiles_m, int tiles_n,
+                       const void* bias, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream, Epilogue epi);
 // the 128-column-tile kernel for a few hundred activation rows, and for any M when K % 64 == 32
 int launch_qmm_mid(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,

@@ -1118,15 +1118,10 @@ bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
 }
 
 // The two-kernel path (qmm_frag.hip: a 16-bit scratch copy of the weights in fragment order, then a lean
-// GEMM) takes the shapes it wins on: at least eight rows of tiles to spread the copy over, tiles that fill
-// four fifths or more of their rounds of the CUs (it does not cut K), and no K cut planned for the fused kernel.
+// GEMM) takes the shapes it wins on: at least eight rows of tiles to spread the copy over.  It cuts K for
+// the tail of the tile sequence by the same plan as the fused kernel.
 bool prefer_frag_path(int64_t M, int64_t N, int64_t K, int gs, int bits) {
-  if (M < 2048 || !qmm_frag_shape_ok(M, N, K, bits) || use_mid_kernel(M, N, K)) return false;
-  const int cus = compute_units();
-  if (plan_tail(M, N, K, period_of(gs), cus).splits > 1) return false;
-  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  const int64_t rounds = (tiles + cus - 1) / cus;
-  return tiles * 5 >= rounds * cus * 4;
+  return M >= 2048 && qmm_frag_shape_ok(M, N, K, bits) && !use_mid_kernel(M, N, K);
 }
 
 size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
@@ -1137,9 +1132,22 @@ size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {
 
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits) {
   const size_t planes = qmm_min_workspace_bytes(M, N, K, gs);
-  if (!prefer_frag_path(M, N, K, gs, bits)) return planes;
-  const size_t copy = qmm_frag_workspace_bytes(N, K);
-  return copy > planes ? copy : planes;
+  return prefer_frag_path(M, N, K, gs, bits) ? qmm_frag_copy_bytes(N, K) + planes : planes;
+}
+
+int launch_tail_reduce(int dtype, const float* planes, int n_whole, int splits, int tiles_m, int tiles_n,
+                       const void* bias, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream, Epilogue epi) {
+  const unsigned blocks = (unsigned)(tiles_m * tiles_n - n_whole) * (BM * BN / 4 / 256);
+  if (dtype == MFQ_BF16) {
+    hipLaunchKernelGGL((tail_reduce_kernel<BF16>), dim3(blocks), dim3(256), 0, stream, planes, n_whole, splits, tiles_m,
+                       tiles_n, (const uint16_t*)bias, (int)M, (int)N, y, (int)(y_dtype == MFQ_F32), epi);
+  } else if (dtype == MFQ_F16) {
+    hipLaunchKernelGGL((tail_reduce_kernel<F16>), dim3(blocks), dim3(256), 0, stream, planes, n_whole, splits, tiles_m,
+                       tiles_n, (const uint16_t*)bias, (int)M, (int)N, y, (int)(y_dtype == MFQ_F32), epi);
+  } else {
+    return MFQ_EDTYPE;
+  }
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
 int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, int64_t N, const void* bias, void* y,
@@ -1167,10 +1175,17 @@ int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
   if (use_mid_kernel(M, N, K))
     return launch_qmm_mid(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
                           workspace_bytes, stream, low_rank, epi);
-  // the two-kernel path where it wins and the caller has brought room for the scratch copy
+  // the two-kernel path where it wins and the caller has brought room for the scratch copy (and, behind it, for
+  // the planes of the K cut: without those the tiles run whole)
   if (!low_rank.R && y_dtype == dtype && workspace && aligned16(workspace) &&
-      workspace_bytes >= qmm_frag_workspace_bytes(N, K) && prefer_frag_path(M, N, K, gs, bits))
-    return launch_qmm_frag(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
+      workspace_bytes >= qmm_frag_copy_bytes(N, K) && prefer_frag_path(M, N, K, gs, bits)) {
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    TailPlan plan = plan_tail(M, N, K, period_of(gs), compute_units());
+    if (plan.splits > 1 && workspace_bytes < qmm_frag_copy_bytes(N, K) + tail_plane_bytes(M, N, plan))
+      plan = TailPlan{(int)tiles, 1};
+    return launch_qmm_frag(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, plan.n_whole,
+                           plan.splits, stream, epi);
+  }
   if (epi.kind != kEpiNone)
     return launch_qmm_epilogue(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,
                                workspace_bytes, stream, epi);

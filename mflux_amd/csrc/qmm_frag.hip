@@ -132,14 +132,44 @@ __device__ inline void mma16(f16x8 a, f16x8 b, f32x4& c) {
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
-template <typename T, bool kEpi>
+// kCut: the instantiation that can cut the tail of the tile sequence along K (apart, so that the code of the
+// shapes that run whole tiles only is what it is without it: the plane store costs the epilogue registers)
+template <typename T, bool kEpi, bool kCut>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void frag_gemm_kernel(
     const uint16_t* __restrict__ x, const char* __restrict__ wfrag, const uint16_t* __restrict__ bias,
-    void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, Epilogue epi) {
+    void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits,
+    float* __restrict__ planes, Epilogue epi) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
-  const int n_items = tiles_m * tiles_n;
-  const int steps = K / BK;  // even, at least 4 (the launcher has checked)
+  const int n_tiles = tiles_m * tiles_n;
+  const int n_items = n_whole + (n_tiles - n_whole) * tail_splits;
+  const int steps_total = K / BK;  // even, at least 4 (the launcher has checked)
+
+  // A work item is (tile, k range): the first n_whole tiles of the sequence run whole; each later one is cut
+  // into tail_splits equal ranges of an even number of steps, every range into a float32 plane of its own
+  // (qmm.hip's K cut: tail_reduce_kernel adds the planes up, rounds, applies bias and epilogue).
+  struct Item {
+    int m0, n0;
+    int first_step, n_steps;
+    int plane;  // -1: the tile is whole and goes to y
+  };
+  auto item_of = [&](int seq) {
+    Item it;
+    int tile = seq;
+    it.first_step = 0;
+    it.n_steps = steps_total;
+    it.plane = -1;
+    if (kCut && seq >= n_whole) {
+      const int e = seq - n_whole;
+      const int tail_tile = e / tail_splits;
+      tile = n_whole + tail_tile;
+      it.n_steps = steps_total / tail_splits;
+      it.first_step = (e - tail_tile * tail_splits) * it.n_steps;
+      it.plane = e;
+    }
+    tile_origin(tile, tiles_m, tiles_n, it.m0, it.n0);
+    return it;
+  };
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
@@ -154,7 +184,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint32_t nb = (uint32_t)min((n0 + wn) / 16 + j, (N - 1) / 16);
-      woff[j] = nb * (uint32_t)steps * (uint32_t)kBlockBytes + (uint32_t)lane * 16u;
+      woff[j] = nb * (uint32_t)steps_total * (uint32_t)kBlockBytes + (uint32_t)lane * 16u;
     }
     // lane l of a direct load lands in LDS at 16 l past the load's base: row l / 8 of the wavefront's eight,
     // 16-byte slot l % 8, which in the swizzled tile holds the row's piece (l % 8) ^ ((row / 2) % 8)
@@ -259,17 +289,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 
   // Fills the pipeline for the tile the cursor is in: x(0) and x(1) into LDS, the
   // fragments of step 0 and the first-pass fragments of step 1.
-  auto prime = [&]() {
+  auto prime = [&](int s0) {  // s0: the item's first step
     const uint32_t w1k = lds_base + (uint32_t)wave * 1024u;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      dma16(xbytes, xoff[i], __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_cur) + 4096u * i);
+      dma16(xbytes + (size_t)s0 * (BK * 2), xoff[i], __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_cur) + 4096u * i);
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-      dma16(xbytes + (size_t)(BK * 2), xoff[i], __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_next) + 4096u * i);
-    load_w(wa, 0, 0);
-    load_w(wa, 1, 0);
-    load_w(wb, 0, 1);
+      dma16(xbytes + (size_t)(s0 + 1) * (BK * 2), xoff[i],
+            __builtin_amdgcn_readfirstlane(w1k + (uint32_t)x_next) + 4096u * i);
+    load_w(wa, 0, s0);
+    load_w(wa, 1, s0);
+    load_w(wb, 0, s0 + 1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both x tiles have landed (the fragments too)
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
@@ -390,48 +421,98 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
                      "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]), "+a"(acc[r + 3][3]));
   };
 
-  bool primed = false;
-  for (int seq = blockIdx.x; seq < n_items; seq += gridDim.x) {
-    int m0, n0;
-    tile_origin(seq, tiles_m, tiles_n, m0, n0);
-    out_base = static_cast<char*>(y) + ((size_t)m0 * N + n0) * 2;
-    out_stride = N;
-    if constexpr (kEpi) {
-      if (epi.kind == kEpiSwiglu) {
-        out_base = static_cast<char*>(y) + ((size_t)m0 * (N / 2) + n0 / 2) * 2;
-        out_stride = N / 2;
+  // A k range's sums as float32 into its dense 256 x 256 plane: the same transpose through the wavefront's
+  // LDS region, 32 rows at a time (a staged row is 64 floats plus 16 bytes), so that every global store
+  // writes complete 256-byte row segments.
+  auto store_plane = [&](float* plane) {
+    constexpr int kStride = 64 * 4 + 16;
+    static_assert(32 * kStride <= kStageBytes, "the float32 staging fits the wavefront's region");
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int c16 = lane_e & 15;
+    const int q = lane_e >> 4;
+    const int lane = lane_e;
+    char* stage = lds + kXBuffers * kTileBytes + wave * kStageBytes;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const int r = 2 * pass + r2;
+          *reinterpret_cast<float4*>(stage + (16 * r2 + c16) * kStride + (16 * j + 4 * q) * 4) =
+              make_float4(acc[r][j][0], acc[r][j][1], acc[r][j][2], acc[r][j][3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int rl = 4 * k + (lane >> 4);
+        const float4 v = *reinterpret_cast<const float4*>(stage + rl * kStride + 16 * (lane & 15));
+        *reinterpret_cast<float4*>(plane + (32 * pass + rl) * BN + wn + 4 * (lane & 15)) = v;
+        if (k & 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if (!primed) {
-      set_prefetch_tile(m0, n0);
-      prime();
-    }
-    const bool has_next = seq + (int)gridDim.x < n_items;
-    m1 = m0, n1 = n0;
-    if (has_next) tile_origin(seq + gridDim.x, tiles_m, tiles_n, m1, n1);
-    const int s_next = has_next ? 0 : steps - 2;  // without a next tile: the last pair again (loaded, not used)
-    settle();
-    // ONE body for every pair of steps, the tile's last included: the accumulators pass through a single
-    // copy of the matrix instructions, so the compiler has no place to move them between register files
-    for (int p = 0; p < steps; p += 2) {
-      const bool last = p == steps - 2;
-      do_step(last, wa, wb, p + 1, last ? s_next : p + 2);
-      do_step(false, wb, wa, last ? s_next : p + 2, last ? s_next + 1 : p + 3);
-    }
-    settle();
-    primed = has_next;
-    if (out_bias) {
-      store_tile_staged(std::true_type{}, m0, n0);
-    } else {
-      store_tile_staged(std::false_type{}, m0, n0);
-    }
+  };
+
+  // The items of this workgroup in sequence: first its whole tiles, then (kCut) its k ranges of tail tiles.
+  // The two kinds run through two instantiations of the same loop, each with one kind of store behind it: with
+  // both stores behind one loop the compiler reads the accumulators ahead of the branch and spills them.
+  bool primed = false;
+  auto run = [&](auto to_planes, int seq, int end) __attribute__((always_inline)) {
+    constexpr bool kPlanes = decltype(to_planes)::value;
+    for (; seq < end; seq += gridDim.x) {
+      const Item item = item_of(seq);
+      const int m0 = item.m0, n0 = item.n0;
+      const int steps = item.n_steps, s0 = item.first_step;
+      if constexpr (!kPlanes) {
+        out_base = static_cast<char*>(y) + ((size_t)m0 * N + n0) * 2;
+        out_stride = N;
+        if constexpr (kEpi) {
+          if (epi.kind == kEpiSwiglu) {
+            out_base = static_cast<char*>(y) + ((size_t)m0 * (N / 2) + n0 / 2) * 2;
+            out_stride = N / 2;
+          }
+        }
+      }
+      if (!primed) {
+        set_prefetch_tile(m0, n0);
+        prime(s0);
+      }
+      const bool has_next = seq + (int)gridDim.x < n_items;
+      Item next = item;
+      if (has_next) next = item_of(seq + gridDim.x);
+      m1 = next.m0, n1 = next.n0;
+      // without a next item: the last pair again (loaded, not used)
+      const int s_next = has_next ? next.first_step : s0 + steps - 2;
+      settle();
+      // ONE body for every pair of steps, the item's last included: the accumulators pass through a single
+      // copy of the matrix instructions, so the compiler has no place to move them between register files
+      for (int p = 0; p < steps; p += 2) {
+        const bool last = p == steps - 2;
+        do_step(last, wa, wb, s0 + p + 1, last ? s_next : s0 + p + 2);
+        do_step(false, wb, wa, last ? s_next : s0 + p + 2, last ? s_next + 1 : s0 + p + 3);
+      }
+      settle();
+      primed = has_next;
+      if constexpr (kPlanes) {
+        store_plane(planes + (size_t)item.plane * (BM * BN));
+      } else if (out_bias) {
+        store_tile_staged(std::true_type{}, m0, n0);
+      } else {
+        store_tile_staged(std::false_type{}, m0, n0);
+      }
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
+      for (int i = 0; i < 16; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
-  }
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+    }
+    return seq;
+  };
+  const int seq_tail = run(std::false_type{}, (int)blockIdx.x, kCut ? n_whole : n_items);
+  if constexpr (kCut) run(std::true_type{}, seq_tail, n_items);
 }
 
 template <typename T, int GS>
@@ -462,28 +543,41 @@ int launch_dequant(const uint32_t* wq, const void* scales, const void* biases, i
   return launch_dequant_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
 }
 
-template <typename T, bool kEpi>
+template <typename T, bool kEpi, bool kCut>
 int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const void* bias, int64_t N, void* y,
-                hipStream_t stream, Epilogue epi) {
-  auto kernel = frag_gemm_kernel<T, kEpi>;
+                int n_whole, int splits, float* planes, hipStream_t stream, Epilogue epi) {
+  auto kernel = frag_gemm_kernel<T, kEpi, kCut>;
   static PerDeviceInt configured;
   if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
   const int tiles_n = (int)((N + BN - 1) / BN);
-  const int n_items = tiles_m * tiles_n;
+  const int n_tail = tiles_m * tiles_n - n_whole;
+  const int n_items = n_whole + n_tail * splits;
   const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x,
-                     (const char*)wfrag, (const uint16_t*)bias, y, (int)M, (int)N, (int)K, tiles_m, tiles_n, epi);
-  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+                     (const char*)wfrag, (const uint16_t*)bias, y, (int)M, (int)N, (int)K, tiles_m, tiles_n, n_whole,
+                     splits, planes, epi);
+  if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
+  if (splits > 1)
+    return launch_tail_reduce(T::code, planes, n_whole, splits, tiles_m, tiles_n, bias, M, N, y, T::code, stream, epi);
+  return MFQ_OK;
 }
 
 template <typename T>
 int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                 const void* bias, int64_t N, int gs, int bits, void* y, void* workspace, hipStream_t stream,
-                 Epilogue epi) {
+                 const void* bias, int64_t N, int gs, int bits, void* y, void* workspace, int n_whole, int splits,
+                 hipStream_t stream, Epilogue epi) {
   if (int rc = launch_dequant<T>(wq, scales, biases, gs, bits, workspace, N, K, stream)) return rc;
-  if (epi.kind != kEpiNone) return launch_gemm<T, true>(x, M, K, workspace, bias, N, y, stream, epi);
-  return launch_gemm<T, false>(x, M, K, workspace, bias, N, y, stream, epi);
+  // the planes of a K cut lie behind the copy
+  float* planes = reinterpret_cast<float*>(static_cast<char*>(workspace) + qmm_frag_copy_bytes(N, K));
+  if (splits > 1) {
+    if (epi.kind != kEpiNone)
+      return launch_gemm<T, true, true>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
+    return launch_gemm<T, false, true>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
+  }
+  if (epi.kind != kEpiNone)
+    return launch_gemm<T, true, false>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
+  return launch_gemm<T, false, false>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
 }
 
 }  // namespace
@@ -495,16 +589,18 @@ bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits) {
          ((N + 15) / 16) * 16 * K < ((int64_t)1 << 31);
 }
 
-size_t qmm_frag_workspace_bytes(int64_t N, int64_t K) { return (size_t)(((N + 15) / 16) * 16 * K * 2); }
+// the copy, rounded up to whole 256 bytes so that what lies behind it is aligned
+size_t qmm_frag_copy_bytes(int64_t N, int64_t K) { return ((size_t)(((N + 15) / 16) * 16 * K * 2) + 255) & ~(size_t)255; }
 
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
-                    hipStream_t stream, Epilogue epi) {
+                    int n_whole, int splits, hipStream_t stream, Epilogue epi) {
   if (!qmm_frag_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+  if (splits > 1 && ((K / BK) % splits || (K / BK / splits) % 2)) return MFQ_EUNSUPPORTED;  // ranges of whole pairs of steps
   if (dtype == MFQ_BF16)
-    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
+    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, epi);
   if (dtype == MFQ_F16)
-    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, stream, epi);
+    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, epi);
   return MFQ_EDTYPE;
 }
 

@@ -339,7 +339,9 @@ def test_qmm_split_k_shapes(oracle, bits, gs, M, K, N):
 def test_qmm_last_round_cut_along_k(oracle, bits):
     """270 tiles on a 256-CU GPU: the first 256 run whole, the 14 of the last
     round are cut along K into float32 planes that a second kernel adds up
-    (ragged M and N, bias; bf16 and float32 output)."""
+    (ragged M and N, bias).  The bf16 call goes through the two-kernel path (its
+    workspace: the 16-bit copy of the weights, then the planes), the call with
+    float32 activations and output through the fused kernel's cut."""
     import mflux_amd
     from gpu_util import to_dev, u32_to_dev
     from mflux_amd import _lib
@@ -347,7 +349,7 @@ def test_qmm_last_round_cut_along_k(oracle, bits):
     o = oracle
     M, K, N = 2200, 2048, 7504
     if torch.cuda.get_device_properties(0).multi_processor_count == 256:
-        assert _lib.load().mfq_qmm_t_workspace_bytes(M, K, N, 64, bits) == 14 * 8 * 256 * 256 * 4
+        assert _lib.load().mfq_qmm_t_workspace_bytes(M, K, N, 64, bits) == N * K * 2 + 14 * 8 * 256 * 256 * 4
     args = _case(o, 34, M, K, N, bits)
     ref = _ref(o, *args, bits)
     _assert_close(_run(o, *args, bits), ref)

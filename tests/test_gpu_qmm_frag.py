@@ -52,7 +52,7 @@ def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_
     M, K, N = 4100, 512, 3208
     need = lib.mfq_qmm_t_workspace_bytes(M, K, N, gs, bits)
     n16 = (N + 15) // 16 * 16
-    assert need == n16 * K * 2, "the shape must take the two-kernel path"
+    assert need == n16 * K * 2, "the shape must take the two-kernel path, uncut"
     x, wq, s, b, bias = _operands(o, 90 + bits + gs, M, K, N, bits, gs, dt, with_bias)
     xd, wd, sd, bd = to_dev(x, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt)
     biasd = None if bias is None else to_dev(bias, dt)
@@ -84,24 +84,55 @@ def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_
     assert not torch.equal(y_fused, torch.zeros_like(y_fused))
 
 
-def test_two_kernel_path_is_chosen_for_full_rounds_only():
-    """The workspace the library asks for tells which path a shape takes: the scratch
-    copy for shapes whose tiles fill their rounds, the K split's planes (or
-    nothing) for the others."""
+def test_workspace_tells_the_path():
+    """The workspace the library asks for tells which path a shape takes: the 16-bit
+    copy (plus the planes of a K cut behind it) from 2048 activation rows on, the
+    fused kernels' planes (or nothing) below."""
     from mflux_amd import _lib
 
     lib = _lib.load()
     if torch.cuda.get_device_properties(0).multi_processor_count != 256:
         pytest.skip("tile counts below are for 256 CUs")
     q = lib.mfq_qmm_t_workspace_bytes
-    assert q(4608, 3072, 21504, 64, 4) == 21504 * 3072 * 2      # FLUX single block, linear1
-    assert q(4608, 15360, 3072, 64, 4) == 3072 * 15360 * 2      # linear2: 216 tiles
-    assert q(4352, 3840, 10240, 64, 8) == 10240 * 3840 * 2      # Z-Image
-    assert q(4096, 3072, 3072, 64, 4) == 0                      # 192 tiles: three quarters of a round, fused kernel
-    assert q(1024, 3072, 21504, 64, 4) < 21504 * 3072 * 2       # four rows of tiles: the copy would not pay
-    planes = q(6889, 3072, 3072, 64, 4)                         # one round + 68 tiles: the fused kernel's K split
-    assert 0 < planes and planes % (256 * 256 * 4) == 0
-    assert q(4608, 3072, 21504, 64, 5) != 21504 * 3072 * 2      # odd bit widths have their own kernel
+    plane = 256 * 256 * 4
+    assert q(4608, 3072, 21504, 64, 4) == 21504 * 3072 * 2      # FLUX single block, linear1: no cut
+    assert q(4608, 15360, 3072, 64, 4) == 3072 * 15360 * 2      # linear2: 216 tiles, no cut
+    assert q(4096, 3072, 3072, 64, 4) == 3072 * 3072 * 2        # 192 tiles: one short round, not worth cutting
+    cut = q(6889, 3072, 3072, 64, 4) - 3072 * 3072 * 2          # one round + 68 tiles: the tail cut along K
+    assert cut > 0 and cut % (68 * plane) == 0
+    assert q(1024, 3072, 21504, 64, 4) % plane == 0             # four rows of tiles: the fused kernel (and its cut)
+    assert q(4608, 3072, 21504, 64, 5) == 0                     # odd bit widths have their own kernel
+
+
+@pytest.mark.parametrize("bits,dtype", [(4, "bf16"), (8, "f16")])
+def test_two_kernel_path_with_a_k_cut(oracle, bits, dtype):
+    """264 tiles on 256 CUs: the eight of the last round are cut along K into planes
+    behind the copy; ragged M; bias; against the float64 oracle, and without the
+    planes' part of the workspace (tiles then run whole) the same bound."""
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    if torch.cuda.get_device_properties(0).multi_processor_count != 256:
+        pytest.skip("tile counts below are for 256 CUs")
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    M, K, N = 2100, 2048, 7440  # 9 x 30 tiles = 270: 14 in the last round; N % 16 == 0, N % 256 != 0
+    need = lib.mfq_qmm_t_workspace_bytes(M, K, N, 64, bits)
+    copy = N * K * 2
+    assert need == copy + 14 * 8 * 256 * 256 * 4
+    x, wq, s, b, bias = _operands(o, 120 + bits, M, K, N, bits, 64, dt, True)
+    xd, wd, sd, bd, biasd = to_dev(x, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt), to_dev(bias, dt)
+    ref = o.quantized_matmul_f64(_to_f64(o, x, dt), wq, s, b, dt, 64, bits, bias_f64=_to_f64(o, bias, dt))
+    row_inf = np.abs(ref).max(axis=-1, keepdims=True)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    for ws_bytes in (need, copy):
+        y = torch.full((M, N), float("nan"), dtype=xd.dtype, device="cuda")
+        assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, 64, bits, xd, wd, sd, bd, biasd, y, ws, ws_bytes) == 0
+        torch.cuda.synchronize()
+        err = np.abs(y.double().cpu().numpy() - ref) / row_inf
+        assert err.max() <= TOL, (ws_bytes, err.max())
 
 
 def test_two_kernel_path_epilogues_and_graph_replay(oracle):
