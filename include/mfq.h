@@ -212,20 +212,22 @@ int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* 
  * cut into ranges that run on different compute units, each range accumulates
  * into its own float32 plane of the workspace, and a second kernel adds the
  * planes, rounds and applies the bias (same two roundings as the fused
- * epilogue).  The opposite shapes -- 4 or 8 bits, 16-bit y, at least 2048
- * activation rows and tiles that fill four fifths or more of their rounds of
- * the compute units, e.g. the single-stream linears of FLUX.1 at M = 4608 --
- * use the workspace for a 16-bit copy of the dequantised weights
- * (round_up(N, 16) * K * 2 bytes, written once per call in the order the matrix
- * instructions consume it) and multiply with a kernel that has no
- * dequantisation in its loop; the copy's values are the ones the fused kernels
- * use (one rounding of fma(code, scale, bias)), the float32 sums run in another
- * order.  mfq_qmm_t_workspace_bytes() returns the size this shape would use on
- * the current device (0: neither applies, pass NULL).  A NULL or smaller
- * workspace is not an error: the call then runs as mfq_qmm_t does (the fused
- * kernel, K not split).  The workspace must be 16-byte aligned; its contents
- * before and after the call are undefined; calls sharing one workspace must be
- * ordered on one stream.
+ * epilogue).  Large calls -- 4 or 8 bits, 16-bit y, K a multiple of 128, at
+ * least 2048 activation rows (where it starts to pay), e.g. the single-stream
+ * linears of FLUX.1 at M = 4608 -- use the workspace first for a 16-bit copy of
+ * the dequantised weights (round_up(N, 16) * K * 2 bytes rounded up to 256,
+ * written once per call in the order the matrix instructions consume it) and
+ * multiply with a kernel that has no dequantisation in its loop; the planes of
+ * a K cut, if the shape has a short last round of tiles, lie behind the copy.
+ * The copy's values are the ones the fused kernels use (one rounding of
+ * fma(code, scale, bias)); the float32 sums run in another order.
+ * mfq_qmm_t_workspace_bytes() returns the size this shape would use on the
+ * current device (0: no use for one, pass NULL).  A NULL or smaller workspace
+ * is not an error: without room for the copy the call runs as mfq_qmm_t does
+ * (the fused kernel, K not split), with room for the copy only its tiles run
+ * whole.  The workspace must be 16-byte aligned; its contents before and after
+ * the call are undefined; calls sharing one workspace must be ordered on one
+ * stream.
  */
 size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits);
 int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
