@@ -47,15 +47,20 @@ def _compile(src: str) -> str:
 ASM_MFMA_KERNELS = {"qmm_frag.hip": "frag_gemm_kernel"}
 
 
-def check_accumulator_moves(src: str) -> int:
+def check_generated_code(src: str) -> int:
     """Compiles `src` to assembly (device side) and checks every kernel named in
     ASM_MFMA_KERNELS: no basic block may hold both a matrix instruction and an
     instruction that moves an accumulator between register files
     (v_accvgpr_read / _write / _mov).  The kernels keep such moves (zeroing, the
     epilogue's reads) in blocks of their own, behind wait states of their own;
     one next to a matrix instruction would read or overwrite a result in flight
-    without the hardware or the compiler noticing.  Returns the number of kernels
-    checked; raises on a finding."""
+    without the hardware or the compiler noticing.  Nor may such a block wait for
+    its loads with a count below 8: the weight fragments are requested a step and
+    a half ahead with at least nine younger requests behind them, and a smaller
+    count means that the compiler's wait counting entered the loop believing
+    loads outstanding that are not, and waits for the newest requests instead
+    (seen once, 20 us per call).  Returns the number of kernels checked; raises
+    on a finding."""
     import re
     import tempfile
 
@@ -78,6 +83,10 @@ def check_accumulator_moves(src: str) -> int:
             if matrix and moves:
                 raise RuntimeError(f"{src}: {m.group(1)} has a basic block with {matrix} matrix instructions and "
                                    f"{moves} accumulator moves")
+            if matrix >= 64:  # the k loop's blocks (the low-rank update's few matrix instructions wait for their own loads)
+                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", block) if int(c) < 8]
+                if short:
+                    raise RuntimeError(f"{src}: {m.group(1)} waits with vmcnt({min(short)}) inside its k loop")
         if not n_matrix:
             raise RuntimeError(f"{src}: {m.group(1)} holds no matrix instruction; the check does not see the kernel")
         checked += 1
@@ -90,7 +99,7 @@ def build_library(verbose: bool = False) -> str:
     """Always recompiles every translation unit, checks the generated code of the
     kernels in ASM_MFMA_KERNELS and relinks libmfq.so."""
     with ThreadPoolExecutor(max_workers=len(SOURCES) + len(ASM_MFMA_KERNELS)) as pool:
-        checks = [pool.submit(check_accumulator_moves, src) for src in ASM_MFMA_KERNELS]
+        checks = [pool.submit(check_generated_code, src) for src in ASM_MFMA_KERNELS]
         objs = list(pool.map(_compile, SOURCES))
         for c in checks:
             c.result()

@@ -351,14 +351,15 @@ int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void*
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits);
 size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // the two-kernel path (qmm_frag.hip): dequantize once into a 16-bit copy in fragment order, then a GEMM on
-// 16x16x32 matrix instructions; 4 and 8 bits, 16-bit y of x's type, epilogues as launch_qmm_epilogue.
+// 16x16x32 matrix instructions; 4 and 8 bits, 16-bit y of x's type, a low-rank update or an epilogue as
+// launch_qmm / launch_qmm_epilogue.
 // workspace (16-byte aligned): qmm_frag_copy_bytes(N, K) for the copy and, behind it, the float32 planes of a
 // K cut (n_whole whole tiles, the others in `splits` ranges of whole pairs of k steps; splits == 1: no cut)
 bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits);
 size_t qmm_frag_copy_bytes(int64_t N, int64_t K);
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
-                    int n_whole, int splits, hipStream_t stream, Epilogue epi);
+                    int n_whole, int splits, hipStream_t stream, LowRank low_rank, Epilogue epi);
 // y tiles = sums of the planes of a K cut (+ bias, epilogue): the second kernel of qmm.hip's and qmm_frag.hip's cut
 int launch_tail_reduce(int dtype, const float* planes, int n_whole, int splits, int tiles_m, int tiles_n,
                        const void* bias, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream, Epilogue epi);

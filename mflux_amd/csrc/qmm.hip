@@ -1177,14 +1177,14 @@ int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                           workspace_bytes, stream, low_rank, epi);
   // the two-kernel path where it wins and the caller has brought room for the scratch copy (and, behind it, for
   // the planes of the K cut: without those the tiles run whole)
-  if (!low_rank.R && y_dtype == dtype && workspace && aligned16(workspace) &&
+  if (y_dtype == dtype && workspace && aligned16(workspace) && !(low_rank.R && epi.kind != kEpiNone) &&
       workspace_bytes >= qmm_frag_copy_bytes(N, K) && prefer_frag_path(M, N, K, gs, bits)) {
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     TailPlan plan = plan_tail(M, N, K, period_of(gs), compute_units());
     if (plan.splits > 1 && workspace_bytes < qmm_frag_copy_bytes(N, K) + tail_plane_bytes(M, N, plan))
       plan = TailPlan{(int)tiles, 1};
     return launch_qmm_frag(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, plan.n_whole,
-                           plan.splits, stream, epi);
+                           plan.splits, stream, low_rank, epi);
   }
   if (epi.kind != kEpiNone)
     return launch_qmm_epilogue(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, workspace,

@@ -134,11 +134,13 @@ __device__ inline void mma16(f16x8 a, f16x8 b, f32x4& c) {
 
 // kCut: the instantiation that can cut the tail of the tile sequence along K (apart, so that the code of the
 // shapes that run whole tiles only is what it is without it: the plane store costs the epilogue registers)
-template <typename T, bool kEpi, bool kCut>
+// kLowRank: lr_rank more k behind the item's own (a LoRA update, see qmm.hip), read straight from memory
+template <typename T, bool kEpi, bool kCut, bool kLowRank>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void frag_gemm_kernel(
     const uint16_t* __restrict__ x, const char* __restrict__ wfrag, const uint16_t* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits,
-    float* __restrict__ planes, Epilogue epi) {
+    float* __restrict__ planes, const uint16_t* __restrict__ lr_t, const uint16_t* __restrict__ lr_bs, int lr_rank,
+    Epilogue epi) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   const int n_tiles = tiles_m * tiles_n;
@@ -301,7 +303,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     load_w(wa, 0, s0);
     load_w(wa, 1, s0);
     load_w(wb, 0, s0 + 1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both x tiles have landed (the fragments too)
+    // both x tiles have landed (the fragments too); as an instruction the compiler sees, so that its own wait
+    // counting enters the loop knowing that nothing is outstanding
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), the other counters at their maxima
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -409,6 +413,46 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
   };
 
+  // The low-rank update: lr_rank more k, whose x side is lr_t [M, lr_rank] and whose weight side is
+  // lr_bs [N, lr_rank], both 16-bit and unquantised.  They are few, so they bypass the pipeline: a lane's
+  // 8 consecutive k of a row are one 16-byte load straight into a matrix fragment (k 32 c + 8 q + 0..7 of
+  // chunk c of 32 on both sides; past the rank, zeros).
+  auto low_rank_steps = [&](int m0, int n0) {
+    int lane_e = lane;  // opaque copy: keeps this per-tile address arithmetic out of the k loop's registers
+    asm volatile("" : "+v"(lane_e));
+    const int c16 = lane_e & 15;
+    const int q = lane_e >> 4;
+    const char* tb = reinterpret_cast<const char*>(lr_t) + 16 * q;
+    const char* bb = reinterpret_cast<const char*>(lr_bs) + 16 * q;
+    const uint32_t pitch = (uint32_t)lr_rank * 2u;  // bytes per row of either matrix
+    uint32_t boff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) boff[j] = (uint32_t)min(n0 + wn + 16 * j + c16, N - 1) * pitch;
+    const uint32_t toff = (uint32_t)min(m0 + c16, M - 1) * pitch;
+    const uint32_t t_last = (uint32_t)(M - 1) * pitch;  // rows 16 r + c16 of the tile: 16 * pitch apart until the clamp
+    const vec8 zero = __builtin_bit_cast(vec8, make_uint4(0u, 0u, 0u, 0u));
+#pragma unroll 1
+    for (uint32_t kb = 0; kb < pitch; kb += 64) {
+      const bool in_rank = kb + 16u * (uint32_t)q < pitch;  // a rank of 16 (mod 32) fills half of the last chunk
+      vec8 wf[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wf[j] = in_rank ? *reinterpret_cast<const vec8*>(bb + boff[j] + kb) : zero;
+#pragma unroll
+      for (int quarter = 0; quarter < 4; ++quarter) {
+        vec8 tf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          tf[i] = in_rank ? *reinterpret_cast<const vec8*>(
+                                tb + min(toff + (uint32_t)(4 * quarter + i) * 16u * pitch, t_last) + kb)
+                          : zero;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) mma16(wf[j], tf[i], acc[4 * quarter + i][j]);
+      }
+    }
+  };
+
   // Every accumulator in its accumulation register, and more wait states than any matrix instruction needs
   // between the instructions in front and behind.
   auto settle = [&]() __attribute__((always_inline)) {
@@ -493,6 +537,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         do_step(last, wa, wb, s0 + p + 1, last ? s_next : s0 + p + 2);
         do_step(false, wb, wa, last ? s_next : s0 + p + 2, last ? s_next + 1 : s0 + p + 3);
       }
+      if constexpr (kLowRank) {
+        if (s0 == 0) low_rank_steps(m0, n0);  // once per tile: by the item that has its first k range
+      }
       settle();
       primed = has_next;
       if constexpr (kPlanes) {
@@ -543,10 +590,10 @@ int launch_dequant(const uint32_t* wq, const void* scales, const void* biases, i
   return launch_dequant_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
 }
 
-template <typename T, bool kEpi, bool kCut>
+template <typename T, bool kEpi, bool kCut, bool kLowRank>
 int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const void* bias, int64_t N, void* y,
-                int n_whole, int splits, float* planes, hipStream_t stream, Epilogue epi) {
-  auto kernel = frag_gemm_kernel<T, kEpi, kCut>;
+                int n_whole, int splits, float* planes, hipStream_t stream, LowRank lr, Epilogue epi) {
+  auto kernel = frag_gemm_kernel<T, kEpi, kCut, kLowRank>;
   static PerDeviceInt configured;
   if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
@@ -556,7 +603,7 @@ int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const vo
   const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
   hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kThreads), kLdsBytes, stream, (const uint16_t*)x,
                      (const char*)wfrag, (const uint16_t*)bias, y, (int)M, (int)N, (int)K, tiles_m, tiles_n, n_whole,
-                     splits, planes, epi);
+                     splits, planes, (const uint16_t*)lr.t, (const uint16_t*)lr.bs, lr.R, epi);
   if (hipGetLastError() != hipSuccess) return MFQ_ELAUNCH;
   if (splits > 1)
     return launch_tail_reduce(T::code, planes, n_whole, splits, tiles_m, tiles_n, bias, M, N, y, T::code, stream, epi);
@@ -566,18 +613,19 @@ int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const vo
 template <typename T>
 int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
                  const void* bias, int64_t N, int gs, int bits, void* y, void* workspace, int n_whole, int splits,
-                 hipStream_t stream, Epilogue epi) {
+                 hipStream_t stream, LowRank lr, Epilogue epi) {
   if (int rc = launch_dequant<T>(wq, scales, biases, gs, bits, workspace, N, K, stream)) return rc;
   // the planes of a K cut lie behind the copy
   float* planes = reinterpret_cast<float*>(static_cast<char*>(workspace) + qmm_frag_copy_bytes(N, K));
-  if (splits > 1) {
-    if (epi.kind != kEpiNone)
-      return launch_gemm<T, true, true>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
-    return launch_gemm<T, false, true>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
-  }
-  if (epi.kind != kEpiNone)
-    return launch_gemm<T, true, false>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
-  return launch_gemm<T, false, false>(x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, epi);
+  auto go = [&](auto e, auto c, auto l) {
+    return launch_gemm<T, decltype(e)::value, decltype(c)::value, decltype(l)::value>(
+        x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, lr, epi);
+  };
+  const std::true_type yes{};
+  const std::false_type no{};
+  if (lr.R) return splits > 1 ? go(no, yes, yes) : go(no, no, yes);  // (no entry point combines update and epilogue)
+  if (epi.kind != kEpiNone) return splits > 1 ? go(yes, yes, no) : go(yes, no, no);
+  return splits > 1 ? go(no, yes, no) : go(no, no, no);
 }
 
 }  // namespace
@@ -594,13 +642,18 @@ size_t qmm_frag_copy_bytes(int64_t N, int64_t K) { return ((size_t)(((N + 15) / 
 
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
-                    int n_whole, int splits, hipStream_t stream, Epilogue epi) {
+                    int n_whole, int splits, hipStream_t stream, LowRank lr, Epilogue epi) {
   if (!qmm_frag_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+  if (lr.R && (epi.kind != kEpiNone || lr.R % 16)) return MFQ_EUNSUPPORTED;
+  // 32-bit byte offsets into the update's operands
+  if ((M + BM) * lr.R >= (int64_t)1 << 31 || (N + BN) * lr.R >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if (splits > 1 && ((K / BK) % splits || (K / BK / splits) % 2)) return MFQ_EUNSUPPORTED;  // ranges of whole pairs of steps
   if (dtype == MFQ_BF16)
-    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, epi);
+    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, lr,
+                              epi);
   if (dtype == MFQ_F16)
-    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, epi);
+    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, lr,
+                             epi);
   return MFQ_EDTYPE;
 }
 

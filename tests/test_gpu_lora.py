@@ -59,12 +59,14 @@ def _assert_close(y, ref, tol=TOL):
     assert worst <= tol, f"max |err| / ||row||inf = {worst:.4g} > {tol}"
 
 
-# M, K, N: the 256 x 256-tile kernel (update inside the epilogue; 2200 x 7504
-# at K = 2048 has its last round cut along K, ragged M and N), the
-# 128-column-tile kernel, the matvec kernels, K an odd multiple of 32
+# M, K, N: the two-kernel path from 2048 rows on (update behind the k loop; 2200 x 7504
+# at K = 2048 has its last round cut along K, ragged M and N; rank 48 fills half of
+# its last chunk of 32), the fused 256 x 256-tile kernel below that (2000 x 5000),
+# the 128-column-tile kernel, the matvec kernels, K an odd multiple of 32
 @pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 32), (8, 128)])
 @pytest.mark.parametrize("M,K,N,R", [
     (2200, 512, 2304, 16), (2200, 2048, 7504, 32), (4608, 1024, 3072, 48), (1000, 1024, 5000, 16),
+    (2000, 1024, 5000, 16),
     (300, 2048, 520, 16), (512, 3072, 768, 64), (100, 512, 1000, 128),
     (1, 3072, 1024, 16), (4, 3072, 1032, 32), (16, 512, 264, 16), (9, 256, 77, 16),
 ])
