@@ -62,18 +62,16 @@ __host__ __device__ inline void tile_origin(int tile, int tiles_m, int tiles_n, 
 }
 
 // ---------------------------------------------------------------------------------------------
-// 1. the scratch copy.  One wavefront per block of 16 rows x 64 k and trip; lane (q, c16) = (lane / 16,
-// lane % 16) owns k [16 q, 16 q + 16) of row c16: 8 (W4) or 16 (W8) bytes of codes, one scale and one bias
-// (16 consecutive k lie in one group), two 16-byte stores, [half][lane].  Consecutive wavefronts take
-// consecutive blocks along K, so a row's codes are read in runs and every store instruction writes 1 KiB.
-// kPair: blocks per wavefront and trip, neighbours along K (K / 64 is a multiple of it), requested together.
+// 1. the scratch copy.  A wavefront takes kPair neighbouring blocks of 16 rows x 64 k per trip (K / 64 is a
+// multiple of kPair); lane (q, c16) = (lane / 16, lane % 16) works on row c16.  Loads are 16 bytes per lane
+// with the four lanes of a row side by side (64 contiguous bytes per row and load: 8-byte loads fetched every
+// 64-byte piece twice and cost a quarter more time), one scale and one bias per load (its 16 or 32 k lie in
+// one group); every store instruction writes whole 256-byte runs of the copy, [block][half][lane].
 template <typename T, int GS, int BITS, int kPair>
 __global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __restrict__ wq,
                                                            const uint16_t* __restrict__ scales,
                                                            const uint16_t* __restrict__ biases,
                                                            char* __restrict__ out, int N, int K, int n_blocks) {
-  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-  using codes_t = std::conditional_t<BITS == 4, u32x2, u32x4>;  // 16 codes
   const int lane = threadIdx.x & (kWave - 1);
   const int c16 = lane & 15, q = lane >> 4;
   const int ks_per_row = K / BK;
@@ -81,35 +79,64 @@ __global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __res
   for (int blk = (blockIdx.x * 4 + threadIdx.x / kWave) * kPair; blk < n_blocks; blk += waves * kPair) {
     const int nb = blk / ks_per_row, ks = blk - nb * ks_per_row;
     const int row = min(nb * 16 + c16, N - 1);  // rows past N repeat the last one; the GEMM never stores their columns
-    codes_t w[kPair];
-    float s[kPair], b[kPair];
+    if constexpr (BITS == 4) {
+      // 16 bytes = 32 codes per load: the lane reads 16-byte piece q + 4 i of its row's kPair * 32 bytes (the
+      // four lanes of a row cover 64 contiguous bytes per load), which holds k 32 (c & 1) .. + 32 of block
+      // c / 2, i.e. the 16-k groups 2 (c & 1) and 2 (c & 1) + 1 of that block, and writes those four pieces
+      constexpr int kLoads = kPair / 2;
+      u32x4 w[kLoads];
+      float s[kLoads], b[kLoads];
 #pragma unroll
-    for (int u = 0; u < kPair; ++u) {
-      const int k0 = (ks + u) * BK + 16 * q;
-      w[u] = __builtin_nontemporal_load(reinterpret_cast<const codes_t*>(wq + ((int64_t)row * K + k0) * BITS / 32));
-      const int64_t g = (int64_t)row * (K / GS) + k0 / GS;
-      s[u] = T::to_f32(scales[g]), b[u] = T::to_f32(biases[g]);
-    }
+      for (int i = 0; i < kLoads; ++i) {
+        const int k0 = ks * BK + 32 * (q + 4 * i);
+        w[i] = *reinterpret_cast<const u32x4*>(wq + ((int64_t)row * K + k0) / 8);
+        const int64_t g = (int64_t)row * (K / GS) + k0 / GS;
+        s[i] = T::to_f32(scales[g]), b[i] = T::to_f32(biases[g]);
+      }
 #pragma unroll
-    for (int u = 0; u < kPair; ++u) {
-      char* dst = out + (int64_t)(blk + u) * kBlockBytes + lane * 16;
+      for (int i = 0; i < kLoads; ++i) {
+        const int c = q + 4 * i;
+        char* dst = out + (int64_t)(blk + (c >> 1)) * kBlockBytes + ((2 * (c & 1)) * 16 + c16) * 16;
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        u32x4 o;
+        for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {  // values 2 p, 2 p + 1 of the half
-          float c0, c1;
-          if constexpr (BITS == 4) {
-            const uint32_t word = w[u][half] >> (8 * p);
-            c0 = (float)(word & 0xfu), c1 = (float)((word >> 4) & 0xfu);
-          } else {
-            const uint32_t word = w[u][2 * half + (p >> 1)] >> (16 * (p & 1));
-            c0 = (float)(word & 0xffu), c1 = (float)((word >> 8) & 0xffu);
+          for (int half = 0; half < 2; ++half) {
+            const uint32_t word = w[i][2 * sub + half];
+            u32x4 o;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+              const float c0 = (float)((word >> (8 * p)) & 0xfu), c1 = (float)((word >> (8 * p + 4)) & 0xfu);
+              o[p] = T::pack2(__builtin_fmaf(c0, s[i], b[i]), __builtin_fmaf(c1, s[i], b[i]));
+            }
+            // plain stores: the GEMM behind reads the copy back through the memory-side cache
+            *reinterpret_cast<u32x4*>(dst + 1024 * half + 256 * sub) = o;
           }
-          o[p] = T::pack2(__builtin_fmaf(c0, s[u], b[u]), __builtin_fmaf(c1, s[u], b[u]));
         }
-        // plain stores: the GEMM behind reads the copy back through the memory-side cache
-        *reinterpret_cast<u32x4*>(dst + 1024 * half) = o;
+      }
+    } else {
+      u32x4 w[kPair];
+      float s[kPair], b[kPair];
+#pragma unroll
+      for (int u = 0; u < kPair; ++u) {
+        const int k0 = (ks + u) * BK + 16 * q;
+        w[u] = *reinterpret_cast<const u32x4*>(wq + ((int64_t)row * K + k0) / 4);
+        const int64_t g = (int64_t)row * (K / GS) + k0 / GS;
+        s[u] = T::to_f32(scales[g]), b[u] = T::to_f32(biases[g]);
+      }
+#pragma unroll
+      for (int u = 0; u < kPair; ++u) {
+        char* dst = out + (int64_t)(blk + u) * kBlockBytes + lane * 16;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          u32x4 o;
+#pragma unroll
+          for (int p = 0; p < 4; ++p) {  // values 2 p, 2 p + 1 of the half
+            const uint32_t word = w[u][2 * half + (p >> 1)] >> (16 * (p & 1));
+            const float c0 = (float)(word & 0xffu), c1 = (float)((word >> 8) & 0xffu);
+            o[p] = T::pack2(__builtin_fmaf(c0, s[u], b[u]), __builtin_fmaf(c1, s[u], b[u]));
+          }
+          *reinterpret_cast<u32x4*>(dst + 1024 * half) = o;
+        }
       }
     }
   }
@@ -566,8 +593,9 @@ template <typename T, int GS>
 int launch_dequant_bits(const uint32_t* wq, const void* scales, const void* biases, int bits, void* out, int64_t N,
                         int64_t K, hipStream_t stream) {
   const int64_t n_blocks = ((N + 15) / 16) * (K / BK);
-  const bool four = (K / BK) % 4 == 0;
-  const int64_t wanted = (n_blocks / (four ? 4 : 2) + 3) / 4;
+  // blocks per wavefront and trip: 4 if that divides the row's count (8 measured slower), else 2
+  const int pair = (K / BK) % 4 == 0 ? 4 : 2;
+  const int64_t wanted = (n_blocks / pair + 3) / 4;
   const int cap = compute_units() * 16;
   const dim3 grid((unsigned)(wanted < cap ? wanted : cap));
   auto launch = [&](auto kernel) {
@@ -575,9 +603,9 @@ int launch_dequant_bits(const uint32_t* wq, const void* scales, const void* bias
                        (char*)out, (int)N, (int)K, (int)n_blocks);
   };
   if (bits == 4) {
-    if (four) launch(dequant_frag_kernel<T, GS, 4, 4>); else launch(dequant_frag_kernel<T, GS, 4, 2>);
+    if (pair == 4) launch(dequant_frag_kernel<T, GS, 4, 4>); else launch(dequant_frag_kernel<T, GS, 4, 2>);
   } else {
-    if (four) launch(dequant_frag_kernel<T, GS, 8, 4>); else launch(dequant_frag_kernel<T, GS, 8, 2>);
+    if (pair == 4) launch(dequant_frag_kernel<T, GS, 8, 4>); else launch(dequant_frag_kernel<T, GS, 8, 2>);
   }
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
