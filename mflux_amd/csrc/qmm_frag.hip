@@ -1,4 +1,4 @@
-// Large-M quantized GEMM in two kernels, for shapes whose 256x256 tiles fill the chip:
+// Large-M quantized GEMM in two kernels (from 2048 activation rows on, where the copy starts to pay):
 //   1. dequant_frag_kernel expands the packed weights ONCE per call into 16-bit values
 //      (w_hat = round(fma(code, scale, bias)), the same single rounding as the fused
 //      kernels) and writes them in the order the matrix instructions consume them:
@@ -9,7 +9,9 @@
 //      wavefronts (one per SIMD, 256 rows x 64 columns each), v_mfma_f32_16x16x32
 //      with the weights as the A operand straight from global memory into registers
 //      and x from global memory straight into LDS (three tiles, no registers in
-//      between), persistent workgroups that prefetch across tile boundaries.
+//      between), persistent workgroups that prefetch across tile boundaries; the
+//      tail of the tile sequence cut along K into float32 planes as in qmm.hip, a
+//      LoRA update as extra k behind the loop, the epilogues of epilogue.h in the store.
 // The fused kernel (qmm.hip) dequantises a weight once per 256 rows of x, M / 256
 // times per call, in the shadow of its matrix instructions; here that vector work is
 // gone from the matrix loop, which is what lets it use the 16-cycle instruction shape
