@@ -181,3 +181,40 @@ def test_two_kernel_path_epilogues_and_graph_replay(oracle):
         assert torch.equal(y_g, plain)
         mflux_amd.quantized_matmul(xd, wd, sd, bd, bits=bits)  # eager work between the replays
         torch.cuda.synchronize()
+
+
+def test_two_kernel_path_is_reproducible_bit_for_bit():
+    """The same call again and again gives the same bits -- whole tiles, a K cut, a
+    LoRA update and an epilogue; with eager work of other shapes in between.  (The
+    matrix instructions of this path are assembly the compiler's hazard checks do
+    not see; a result read or overwritten in flight would show up here as a
+    difference between runs.)"""
+    import mflux_amd
+
+    torch.manual_seed(11)
+    dev = "cuda"
+    cases = [(4608, 1024, 3072, 4, 0), (2100, 2048, 7440, 8, 0), (4608, 512, 3328, 4, 32), (4400, 3072, 21504, 4, 0)]
+    for M, K, N, bits, rank in cases:
+        x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+        w = (torch.randn(N, K, device=dev) * 0.02).to(torch.bfloat16)
+        bias = torch.randn(N, device=dev, dtype=torch.bfloat16)
+        wq, s, b = mflux_amd.quantize(w, 64, bits)
+        low_rank = None
+        if rank:
+            low_rank = (torch.randn(M, rank, device=dev, dtype=torch.bfloat16),
+                        (torch.randn(N, rank, device=dev) * 0.05).to(torch.bfloat16))
+        other = torch.randn(300, K, device=dev, dtype=torch.bfloat16)
+
+        def plain():
+            return mflux_amd.quantized_matmul(x, wq, s, b, bits=bits, bias=bias, low_rank=low_rank)
+
+        def gelu():
+            return mflux_amd.quantized_matmul_epilogue(x, wq, s, b, epilogue="gelu", bits=bits, bias=bias)
+
+        for fn in (plain,) if rank else (plain, gelu):
+            first = fn()
+            for i in range(12 if M * K * N < 1e11 else 4):
+                mflux_amd.quantized_matmul(other, wq, s, b, bits=bits)  # another kernel in between
+                again = fn()
+                assert torch.equal(first, again), (M, K, N, bits, rank, fn.__name__, i)
+        assert bool(torch.isfinite(first).all())
