@@ -49,18 +49,29 @@ ASM_MFMA_KERNELS = {"qmm_frag.hip": "frag_gemm_kernel"}
 
 def check_generated_code(src: str) -> int:
     """Compiles `src` to assembly (device side) and checks every kernel named in
-    ASM_MFMA_KERNELS: no basic block may hold both a matrix instruction and an
-    instruction that moves an accumulator between register files
-    (v_accvgpr_read / _write / _mov).  The kernels keep such moves (zeroing, the
-    epilogue's reads) in blocks of their own, behind wait states of their own;
-    one next to a matrix instruction would read or overwrite a result in flight
-    without the hardware or the compiler noticing.  Nor may such a block wait for
-    its loads with a count below 8: the weight fragments are requested a step and
-    a half ahead with at least nine younger requests behind them, and a smaller
-    count means that the compiler's wait counting entered the loop believing
-    loads outstanding that are not, and waits for the newest requests instead
-    (seen once, 20 us per call).  Returns the number of kernels checked; raises
-    on a finding."""
+    ASM_MFMA_KERNELS for what neither the hardware nor the compiler's hazard
+    recognizer (which does not see matrix instructions written as assembly)
+    would catch, along the listing and across block boundaries:
+    (1) a read of an accumulation register (v_accvgpr_read, the source of a
+    v_accvgpr_mov) or a write of one from outside the matrix pipeline
+    (v_accvgpr_write, the destination of a _mov) must lie at least 24
+    instructions behind the last matrix instruction that wrote that register:
+    the kernels touch accumulators either behind wait states of their own, or
+    (the first pass of a tile, which stores the previous one) some sixty matrix
+    instructions after the register's last update;
+    (2) a matrix instruction that adds to a register must lie at least 4
+    instructions behind a write of that register from outside the pipeline;
+    (3) the body of the k loop may not wait for its loads with a count below 8:
+    the weight fragments are requested a step and a half ahead with at least
+    nine younger requests behind them, and a smaller count means that the
+    compiler's wait counting entered the loop believing loads outstanding that
+    are not, and waits for the newest requests instead (seen once, 20 us per
+    call);
+    (4) a kernel may spill at most 48 registers (the kernels use all 512 and
+    spill a dozen or two outside the k loop; the compiler's choices around the
+    assembly have tipped over into hundreds, with accumulators moved between
+    the register files, on small changes to the source).
+    Returns the number of kernels checked; raises on a finding."""
     import re
     import tempfile
 
@@ -78,17 +89,45 @@ def check_generated_code(src: str) -> int:
         for block in re.split(r"\n\.LBB[0-9_]+:", body):
             ops = [ln.split()[0] for ln in block.split("\n") if ln.strip() and not ln.strip().startswith((";", "."))]
             matrix = sum(op.startswith("v_mfma") for op in ops)
-            moves = sum(op.startswith("v_accvgpr") for op in ops)
             n_matrix += matrix
-            if matrix and moves:
-                raise RuntimeError(f"{src}: {m.group(1)} has a basic block with {matrix} matrix instructions and "
-                                   f"{moves} accumulator moves")
-            if matrix >= 64:  # the k loop's blocks (the low-rank update's few matrix instructions wait for their own loads)
-                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", block) if int(c) < 8]
+            if matrix >= 128:  # the k loop's body (an item's first step and the low-rank update are blocks of fewer)
+                upto = block[:block.rindex("v_mfma")]  # behind the last one the block may run on into an epilogue
+                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", upto) if int(c) < 8]
                 if short:
                     raise RuntimeError(f"{src}: {m.group(1)} waits with vmcnt({min(short)}) inside its k loop")
+        by_matrix = []  # per instruction: the register range a matrix instruction wrote, else None
+        by_move = []    # per instruction: the register a write from outside the pipeline went to, else None
+        for ln in body.split("\n"):
+            ln = ln.strip()
+            if not ln or ln.startswith((";", ".")):
+                continue
+            op = ln.split()[0]
+            wrote, moved = None, None
+            if op.startswith("v_mfma"):
+                ranges = [(int(a), int(b)) for a, b in re.findall(r"a\[(\d+):(\d+)\]", ln)]
+                wrote = ranges[0]
+                if len(ranges) > 1:  # the addend
+                    lo, hi = ranges[-1]
+                    if any(r is not None and lo <= r <= hi for r in by_move[-4:]):
+                        raise RuntimeError(f"{src}: {m.group(1)}: a matrix instruction adds to a[{lo}:{hi}] within 4 "
+                                           f"instructions of a write to it")
+            elif op.startswith("v_accvgpr"):
+                regs = [int(r) for r in re.findall(r"\ba(\d+)\b", ln)]
+                if op.startswith("v_accvgpr_write"):
+                    moved = regs[0]
+                elif op.startswith("v_accvgpr_mov"):
+                    moved = regs[0]
+                for reg in regs:
+                    if any(r is not None and r[0] <= reg <= r[1] for r in by_matrix[-24:]):
+                        raise RuntimeError(f"{src}: {m.group(1)} touches a{reg} within 24 instructions of a matrix "
+                                           f"instruction that writes it")
+            by_matrix.append(wrote)
+            by_move.append(moved)
         if not n_matrix:
             raise RuntimeError(f"{src}: {m.group(1)} holds no matrix instruction; the check does not see the kernel")
+        spills = re.search(r"\.name:\s+%s\n(?:.*\n)*?\s*\.vgpr_spill_count:\s*(\d+)" % re.escape(m.group(1)), text)
+        if spills is None or int(spills.group(1)) > 48:
+            raise RuntimeError(f"{src}: {m.group(1)} spills {spills and spills.group(1)} registers (at most 48 expected)")
         checked += 1
     if not checked:
         raise RuntimeError(f"{src}: no kernel named *{ASM_MFMA_KERNELS[src]}* found")

@@ -149,16 +149,31 @@ __global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __res
 //
 // The matrix instruction with its sum accumulated in place, as assembly: the compiler is free to give an
 // intrinsic's four result registers another place than its addend's, and with every one of the 256
-// accumulation registers holding part of the tile it then rotates accumulators through the vector
-// registers around every instruction.  Stated with the result tied to the addend, the instruction is
-// opaque to the compiler's hazard recognizer, so the kernel keeps every other instruction that touches
-// an accumulator (zeroing, the epilogue's reads) in other basic blocks than the matrix instructions and
-// separates them by settle() below; the build checks the generated code for that (_build.py).
-__device__ inline void mma16(bf16x8 a, bf16x8 b, f32x4& c) {
+// accumulation registers holding part of the tile it then rotates accumulators through the vector registers
+// around every instruction.  Stated with the result tied to the addend, the instruction is opaque to the
+// compiler's hazard recognizer, so the kernel keeps zeroing and the epilogue's reads in other basic blocks
+// than the matrix instructions, separated from them by settle() below, and reads an accumulator between
+// matrix instructions only where the last one on that register is some sixty instructions behind (acc_read);
+// the build checks the generated code for both (_build.py).
+__device__ __forceinline__ void mma16(bf16x8 a, bf16x8 b, f32x4& c) {
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-__device__ inline void mma16(f16x8 a, f16x8 b, f32x4& c) {
+__device__ __forceinline__ void mma16(f16x8 a, f16x8 b, f32x4& c) {
   asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+// The first matrix instruction of a tile: the product alone, whatever the registers held.  Stated as an
+// update all the same, so that the tile's sums stay in the registers the previous tile's were in.
+__device__ __forceinline__ void mma16_first(bf16x8 a, bf16x8 b, f32x4& c) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mma16_first(f16x8 a, f16x8 b, f32x4& c) {
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
+}
+// An accumulator as four floats in vector registers, read HERE: the empty statement gives the accumulator a
+// new name at this point, so that the reads cannot be hoisted to where all of them would be live at once.
+__device__ __forceinline__ void acc_read(f32x4& c, float (&v)[4]) {
+  asm volatile("" : "+a"(c));
+  v[0] = c[0], v[1] = c[1], v[2] = c[2], v[3] = c[3];
 }
 
 // kCut: the instantiation that can cut the tail of the tile sequence along K (apart, so that the code of the
@@ -259,6 +274,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       set[2 * j + half] = *reinterpret_cast<const vec8*>(wfrag + (size_t)step * kBlockBytes + woff[j] + 1024 * half);
   };
 
+  char* drain_out = nullptr;  // the previous tile's place in y while the accumulators still hold it
+  bool pending = false;       // they do
   int m1 = 0, n1 = 0;  // the tile the prefetch cursor moves to in the middle of a tile's last-but-one step
   // Step p = two passes of 64 matrix instructions (16 row blocks x 4 column tiles).  Behind them: every
   // fourth slot the LDS read of the x fragment three row blocks ahead; in the first pass the request for
@@ -267,8 +284,53 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // the x tile of step p+2 into the LDS tile that step p-1 read -- one load every eighth (weights) or
   // seventh (x) slot rather than in a burst, which measured 1 % faster.  s_h1 / s_h0: the steps (counted inside
   // the cursor's tile) those requests are for; `sw`: the cursor enters the next tile between the passes.
-  auto do_step = [&](bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
+  //
+  // kDrain 3: the first step of an item; its first pass writes the bare products (no addend, so nothing is
+  // zeroed between items).
+  // kDrain 1: the same, and the accumulators may still hold the PREVIOUS tile (drain_out: its
+  // place in y), and this is the first step of the next one.  Its first pass then empties them as it goes: the
+  // matrix instructions of row block r write the bare product (no addend, so nothing is zeroed either) while
+  // the slots behind them round row block r+1 to 16 bits and write it into the wavefront's staging region,
+  // 32 rows (two row blocks) to a half; a filled half is read back as whole 128-byte row segments during the
+  // next row block and stored during the one after, while the other half fills.  Every read of an accumulator
+  // is at least 60 matrix instructions behind the one that wrote it.  The pass is issue-bound (about twice
+  // its usual time) instead of the 6 us a tile's stores cost with the matrix pipeline idle.
+  auto do_step = [&](auto drain_mode, bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
       __attribute__((always_inline)) {
+    constexpr int kDrain = decltype(drain_mode)::value;
+    constexpr int kHalfBytes = kStageBytes / 2;
+    static_assert(32 * kStageStride <= kHalfBytes, "32 staged rows to a half");
+    char* st_w = nullptr;
+    const char* st_r = nullptr;
+    uint32_t out_off = 0;
+    u32x4 rb[4];
+    auto drain_part = [&](int r, int j) __attribute__((always_inline)) {
+      uint32_t pk[2];
+      float v[4];
+      acc_read(acc[r][j], v);
+#pragma unroll
+      for (int c = 0; c < 2; ++c) pk[c] = T::pack2(v[2 * c], v[2 * c + 1]);
+      *reinterpret_cast<uint2*>(st_w + ((r >> 1) & 1) * kHalfBytes + 16 * (r & 1) * kStageStride + 32 * j) =
+          make_uint2(pk[0], pk[1]);
+    };
+    auto drain_read = [&](int u, int k) __attribute__((always_inline)) {  // rows 32 u + 8 k + lane / 8
+      rb[k] = *reinterpret_cast<const u32x4*>(st_r + (u & 1) * kHalfBytes + 8 * k * kStageStride);
+    };
+    auto drain_store = [&](int u, int k) __attribute__((always_inline)) {
+      char* rows = drain_out + (size_t)(32 * u + 8 * k) * ((size_t)N * 2);
+      if (pending) *reinterpret_cast<u32x4*>(rows + out_off) = rb[k];
+    };
+    if constexpr (kDrain == 1) {
+      int lane_e = lane;  // opaque copy: keeps this per-tile address arithmetic out of the k loop's registers
+      asm volatile("" : "+v"(lane_e));
+      char* stage = lds + kXBuffers * kTileBytes + wave * kStageBytes;
+      st_w = stage + (lane_e & 15) * kStageStride + 8 * (lane_e >> 4);
+      st_r = stage + (lane_e >> 3) * kStageStride + 16 * (lane_e & 7);
+      out_off = ((uint32_t)(lane_e >> 3) * (uint32_t)N + (uint32_t)wn + 8u * (uint32_t)(lane_e & 7)) * 2u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) drain_part(0, j);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     const char* xs = lds + x_cur;
     const uint32_t fill = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)x_fill + (uint32_t)wave * 1024u);
     vec8 xf[4];
@@ -289,7 +351,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         for (int j = 0; j < 4; ++j) {
           const int m = 4 * r + j;
           const int g = 16 * half + r;
-          mma16(now[2 * j + half], xf[g & 3], acc[r][j]);
+          if (kDrain != 0 && half == 0) {
+            mma16_first(now[2 * j + half], xf[g & 3], acc[r][j]);
+            if constexpr (kDrain == 1) {
+              if (r + 1 < 16) drain_part(r + 1, j);
+              if (r & 1) drain_read(r >> 1, j);
+              if (r >= 2 && !(r & 1)) drain_store((r - 2) >> 1, j);
+            }
+          } else {
+            mma16(now[2 * j + half], xf[g & 3], acc[r][j]);
+            if (kDrain == 1 && r == 0) drain_store(7, j);
+          }
           if (j == 0 && g + 3 < 32) read_frag(g + 3);
           if ((m & 7) == 2 && m < 32) {
             const int j1 = m >> 3;
@@ -494,6 +566,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
                      "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]), "+a"(acc[r + 3][3]));
   };
 
+  // Behind an epilogue: new values for the accumulators (the next item's first step overwrites them anyway), so
+  // that the compiler has nothing of the old ones to keep alive across the stores.
+  auto forget = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[r][j][e] = 0.f;
+  };
+
   // A k range's sums as float32 into its dense 256 x 256 plane: the same transpose through the wavefront's
   // LDS region, 32 rows at a time (a staged row is 64 floats plus 16 bytes), so that every global store
   // writes complete 256-byte row segments.
@@ -558,19 +641,38 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       m1 = next.m0, n1 = next.n0;
       // without a next item: the last pair again (loaded, not used)
       const int s_next = has_next ? next.first_step : s0 + steps - 2;
-      settle();
-      // ONE body for every pair of steps, the item's last included: the accumulators pass through a single
-      // copy of the matrix instructions, so the compiler has no place to move them between register files
-      for (int p = 0; p < steps; p += 2) {
+      // The first step of an item starts the sums (and stores the previous tile if that is still in the
+      // accumulators); ONE body for every later pair of steps, the item's last included: the accumulators pass
+      // through a single copy of those matrix instructions, so the compiler has no place to move them between
+      // register files.
+      if (!pending) settle();
+      {
+        const bool last = steps == 2;
+        const int s_even = last ? s_next : s0 + 2;
+        do_step(std::integral_constant<int, (kPlanes || kEpi) ? 3 : 1>{}, last, wa, wb, s0 + 1, s_even);
+        do_step(std::integral_constant<int, 0>{}, false, wb, wa, s_even, last ? s_next + 1 : s0 + 3);
+      }
+      for (int p = 2; p < steps; p += 2) {
         const bool last = p == steps - 2;
-        do_step(last, wa, wb, s0 + p + 1, last ? s_next : s0 + p + 2);
-        do_step(false, wb, wa, last ? s_next : s0 + p + 2, last ? s_next + 1 : s0 + p + 3);
+        const int s_even = last ? s_next : s0 + p + 2;
+        do_step(std::integral_constant<int, 0>{}, last, wa, wb, s0 + p + 1, s_even);
+        do_step(std::integral_constant<int, 0>{}, false, wb, wa, s_even, last ? s_next + 1 : s0 + p + 3);
       }
       if constexpr (kLowRank) {
         if (s0 == 0) low_rank_steps(m0, n0);  // once per tile: by the item that has its first k range
       }
-      settle();
       primed = has_next;
+      if constexpr (!kPlanes && !kEpi) {
+        // A tile with all of its rows and columns inside y and no output bias, followed by another whole
+        // tile, leaves its sums in the accumulators: the next tile's first step stores them.
+        if (seq + (int)gridDim.x < end && m0 + BM <= M && n0 + BN <= N && !out_bias) {
+          drain_out = out_base;
+          pending = true;
+          continue;
+        }
+      }
+      pending = false;
+      settle();
       if constexpr (kPlanes) {
         store_plane(planes + (size_t)item.plane * (BM * BN));
       } else if (out_bias) {
@@ -578,12 +680,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       } else {
         store_tile_staged(std::false_type{}, m0, n0);
       }
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+      forget();
     }
     return seq;
   };

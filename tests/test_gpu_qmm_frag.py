@@ -136,6 +136,41 @@ def test_two_kernel_path_with_a_k_cut(oracle, bits, dtype):
         assert err.max() <= TOL, (ws_bytes, err.max())
 
 
+@pytest.mark.parametrize("bits,dtype,M,K,N", [(4, "bf16", 4608, 256, 7680), (8, "f16", 2100, 512, 7688)])
+def test_two_kernel_path_deferred_stores(oracle, bits, dtype, M, K, N):
+    """More tiles than CUs, run whole (the workspace holds the copy only): a tile without
+    an output bias that lies inside y and has a successor on its workgroup is stored by
+    that successor's first step.  A bias of -0.0 changes no bit of the result but takes
+    every tile through the immediate epilogue, so the two calls must agree bit for bit;
+    the float64 oracle bounds both.  The second shape has ragged edges in M and N (whose
+    tiles are never deferred) next to deferred interior tiles."""
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert ((M + 255) // 256) * ((N + 255) // 256) > cus + 16
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    x, wq, s, b, _ = _operands(o, 140 + bits, M, K, N, bits, 64, dt, False)
+    xd, wd, sd, bd = to_dev(x, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt)
+    neg_zero = torch.full((N,), -0.0, dtype=xd.dtype, device="cuda")
+    copy = (N + 15) // 16 * 16 * K * 2
+    ws = torch.empty(copy, dtype=torch.uint8, device="cuda")
+    ys = []
+    for biasd in (None, neg_zero):
+        y = torch.full((M, N), float("nan"), dtype=xd.dtype, device="cuda")
+        assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, 64, bits, xd, wd, sd, bd, biasd, y, ws, copy) == 0
+        torch.cuda.synchronize()
+        ys.append(y)
+    assert torch.equal(ys[0].view(torch.int16), ys[1].view(torch.int16))
+    ref = o.quantized_matmul_f64(_to_f64(o, x, dt), wq, s, b, dt, 64, bits)
+    row_inf = np.abs(ref).max(axis=-1, keepdims=True)
+    err = np.abs(ys[0].double().cpu().numpy() - ref) / row_inf
+    assert err.max() <= TOL, err.max()
+
+
 def test_two_kernel_path_epilogues_and_graph_replay(oracle):
     """GELU from a column on, gate * y + residual and SwiGLU through the two-kernel
     path against the composed reference, and a captured call replayed bit for bit."""
