@@ -76,6 +76,16 @@ def test_low_rank_update_vs_f64(oracle, bits, gs, M, K, N, R):
     _assert_close(_run(o, *args, bits, gs, o.BF16), _ref(o, *args, bits, gs, o.BF16))
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_low_rank_update_with_deferred_tile_stores(oracle, bits):
+    """540 tiles on 256 CUs without an output bias: every workgroup's first tile is
+    stored by the first step of its second one, after the update's matrix
+    instructions have added to it; the last 28 tiles are cut along K."""
+    o = oracle
+    args = _operands(o, 54, 4608, 256, 7680, bits, 64, 16, with_bias=False)
+    _assert_close(_run(o, *args, bits, 64, o.BF16), _ref(o, *args, bits, 64, o.BF16))
+
+
 def test_low_rank_update_k_odd_multiple_of_32(oracle):
     o = oracle
     args = _operands(o, 51, 300, 96, 200, 4, 32, 16)
