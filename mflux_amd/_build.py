@@ -61,9 +61,10 @@ def check_generated_code(src: str) -> int:
     instructions after the register's last update;
     (2) a matrix instruction that adds to a register must lie at least 4
     instructions behind a write of that register from outside the pipeline;
-    (3) the body of the k loop may not wait for its loads with a count below 8:
-    the weight fragments are requested a step and a half ahead with at least
-    nine younger requests behind them, and a smaller count means that the
+    (3) the body of the k loop may not wait for its loads with a count below 8
+    (6 with three column tiles per wavefront instead of four): the weight
+    fragments are requested a step and a half ahead with at least nine (six)
+    younger requests behind them, and a smaller count means that the
     compiler's wait counting entered the loop believing loads outstanding that
     are not, and waits for the newest requests instead (seen once, 20 us per
     call);
@@ -86,13 +87,15 @@ def check_generated_code(src: str) -> int:
     for m in re.finditer(r"^(\S*%s\S*):" % re.escape(ASM_MFMA_KERNELS[src]), text, re.M):
         body = text[m.end():text.index(".Lfunc_end", m.end())]
         n_matrix = 0
+        col_tiles = re.search(r"ELi(\d)EEEv", m.group(1))  # the kernel's last template argument: column tiles per wavefront
+        least = 2 * int(col_tiles.group(1)) if col_tiles else 8
         for block in re.split(r"\n\.LBB[0-9_]+:", body):
             ops = [ln.split()[0] for ln in block.split("\n") if ln.strip() and not ln.strip().startswith((";", "."))]
             matrix = sum(op.startswith("v_mfma") for op in ops)
             n_matrix += matrix
             if matrix >= 128:  # the k loop's body (an item's first step and the low-rank update are blocks of fewer)
                 upto = block[:block.rindex("v_mfma")]  # behind the last one the block may run on into an epilogue
-                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", upto) if int(c) < 8]
+                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", upto) if int(c) < least]
                 if short:
                     raise RuntimeError(f"{src}: {m.group(1)} waits with vmcnt({min(short)}) inside its k loop")
         by_matrix = []  # per instruction: the register range a matrix instruction wrote, else None

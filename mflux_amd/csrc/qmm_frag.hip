@@ -179,7 +179,10 @@ __device__ __forceinline__ void acc_read(f32x4& c, float (&v)[4]) {
 // kCut: the instantiation that can cut the tail of the tile sequence along K (apart, so that the code of the
 // shapes that run whole tiles only is what it is without it: the plane store costs the epilogue registers)
 // kLowRank: lr_rank more k behind the item's own (a LoRA update, see qmm.hip), read straight from memory
-template <typename T, bool kEpi, bool kCut, bool kLowRank>
+// kJ: column tiles of 16 per wavefront, i.e. tiles of 256 rows x 64 kJ columns: 4, or 3 (192 columns) for
+//     shapes whose 192-column tiles fit one round of workgroups (a quarter less work per workgroup than the
+//     256-column tiles of the same round); without epilogue or K cut
+template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void frag_gemm_kernel(
     const uint16_t* __restrict__ x, const char* __restrict__ wfrag, const uint16_t* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits,
@@ -187,6 +190,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     Epilogue epi) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
+  static_assert(kJ == 4 || (kJ == 3 && !kEpi && !kCut), "192-column tiles: plain whole tiles only");
+  constexpr int kBN = 64 * kJ;  // columns of a tile
   const int n_tiles = tiles_m * tiles_n;
   const int n_items = n_whole + (n_tiles - n_whole) * tail_splits;
   const int steps_total = K / BK;  // even, at least 4 (the launcher has checked)
@@ -214,21 +219,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       it.plane = e;
     }
     tile_origin(tile, tiles_m, tiles_n, it.m0, it.n0);
+    it.n0 = it.n0 / BN * kBN;
     return it;
   };
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
-  const int wn = wave * 64;
+  const int wn = wave * (16 * kJ);
   const int c16 = lane & 15;
   const int q = lane >> 4;
 
   // Per-lane byte offsets of the tile the PREFETCH cursor is in: the blocks of the wavefront's four column tiles
   // (16 columns each; blocks past N repeat the last one) and the lane's eight x pieces (rows past M clamped).
-  uint32_t woff[4], xoff[8];
+  uint32_t woff[kJ], xoff[8];
   auto set_prefetch_tile = [&](int m0, int n0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kJ; ++j) {
       const uint32_t nb = (uint32_t)min((n0 + wn) / 16 + j, (N - 1) / 16);
       woff[j] = nb * (uint32_t)steps_total * (uint32_t)kBlockBytes + (uint32_t)lane * 16u;
     }
@@ -256,21 +262,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
   for (int half = 0; half < 2; ++half) rd_slot[half] = swz(c16, 2 * q + half);
 
-  vec8 wa[8], wb[8];  // weight fragments of the even / odd steps: [2 j + pass], column tile j
+  vec8 wa[2 * kJ], wb[2 * kJ];  // weight fragments of the even / odd steps: [2 j + pass], column tile j
   char* out_base = static_cast<char*>(y);
   int out_stride = N;
   const uint16_t* out_bias = bias;
-  f32x4 acc[16][4];   // [r][j][e]: row 16 r + c16, column 16 j + 4 q + e of the wavefront's 256 x 64 block
+  f32x4 acc[16][kJ];  // [r][j][e]: row 16 r + c16, column 16 j + 4 q + e of the wavefront's 256 x 16 kJ block
 #pragma unroll
   for (int i = 0; i < 16; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kJ; ++j)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-  auto load_w = [&](vec8 (&set)[8], int half, int step) __attribute__((always_inline)) {
+  auto load_w = [&](vec8 (&set)[2 * kJ], int half, int step) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kJ; ++j)
       set[2 * j + half] = *reinterpret_cast<const vec8*>(wfrag + (size_t)step * kBlockBytes + woff[j] + 1024 * half);
   };
 
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // next row block and stored during the one after, while the other half fills.  Every read of an accumulator
   // is at least 60 matrix instructions behind the one that wrote it.  The pass is issue-bound (about twice
   // its usual time) instead of the 6 us a tile's stores cost with the matrix pipeline idle.
-  auto do_step = [&](auto drain_mode, bool sw, vec8 (&now)[8], vec8 (&other)[8], int s_h1, int s_h0)
+  auto do_step = [&](auto drain_mode, bool sw, vec8 (&now)[2 * kJ], vec8 (&other)[2 * kJ], int s_h1, int s_h0)
       __attribute__((always_inline)) {
     constexpr int kDrain = decltype(drain_mode)::value;
     constexpr int kHalfBytes = kStageBytes / 2;
@@ -303,7 +309,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     char* st_w = nullptr;
     const char* st_r = nullptr;
     uint32_t out_off = 0;
-    u32x4 rb[4];
+    uint32_t rd_off[kJ], gl_off[kJ];  // 192-column tiles: the lane's piece of each read-back and store of a half
+    u32x4 rb[kJ];
     auto drain_part = [&](int r, int j) __attribute__((always_inline)) {
       uint32_t pk[2];
       float v[4];
@@ -313,22 +320,38 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       *reinterpret_cast<uint2*>(st_w + ((r >> 1) & 1) * kHalfBytes + 16 * (r & 1) * kStageStride + 32 * j) =
           make_uint2(pk[0], pk[1]);
     };
-    auto drain_read = [&](int u, int k) __attribute__((always_inline)) {  // rows 32 u + 8 k + lane / 8
-      rb[k] = *reinterpret_cast<const u32x4*>(st_r + (u & 1) * kHalfBytes + 8 * k * kStageStride);
+    // a half holds 32 rows of 2 kJ 16-byte pieces; read-back k of kJ takes pieces 64 k + lane in row-major
+    // order: with 8 pieces to a row that is row 8 k + lane / 8, piece lane % 8
+    auto drain_read = [&](int u, int k) __attribute__((always_inline)) {
+      if constexpr (kJ == 4) {
+        rb[k] = *reinterpret_cast<const u32x4*>(st_r + (u & 1) * kHalfBytes + 8 * k * kStageStride);
+      } else {
+        rb[k] = *reinterpret_cast<const u32x4*>(st_r + (u & 1) * kHalfBytes + rd_off[k]);
+      }
     };
     auto drain_store = [&](int u, int k) __attribute__((always_inline)) {
-      char* rows = drain_out + (size_t)(32 * u + 8 * k) * ((size_t)N * 2);
-      if (pending) *reinterpret_cast<u32x4*>(rows + out_off) = rb[k];
+      char* rows = drain_out + (size_t)(32 * u + (kJ == 4 ? 8 * k : 0)) * ((size_t)N * 2);
+      if (pending) *reinterpret_cast<u32x4*>(rows + (kJ == 4 ? out_off : gl_off[k])) = rb[k];
     };
     if constexpr (kDrain == 1) {
       int lane_e = lane;  // opaque copy: keeps this per-tile address arithmetic out of the k loop's registers
       asm volatile("" : "+v"(lane_e));
       char* stage = lds + kXBuffers * kTileBytes + wave * kStageBytes;
       st_w = stage + (lane_e & 15) * kStageStride + 8 * (lane_e >> 4);
-      st_r = stage + (lane_e >> 3) * kStageStride + 16 * (lane_e & 7);
-      out_off = ((uint32_t)(lane_e >> 3) * (uint32_t)N + (uint32_t)wn + 8u * (uint32_t)(lane_e & 7)) * 2u;
+      if constexpr (kJ == 4) {
+        st_r = stage + (lane_e >> 3) * kStageStride + 16 * (lane_e & 7);
+        out_off = ((uint32_t)(lane_e >> 3) * (uint32_t)N + (uint32_t)wn + 8u * (uint32_t)(lane_e & 7)) * 2u;
+      } else {
+        st_r = stage;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) drain_part(0, j);
+        for (int k = 0; k < kJ; ++k) {
+          const uint32_t idx = 64u * k + (uint32_t)lane_e, row = idx / (2 * kJ), piece = idx - row * (2 * kJ);
+          rd_off[k] = row * kStageStride + 16u * piece;
+          gl_off[k] = (row * (uint32_t)N + (uint32_t)wn + 8u * piece) * 2u;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kJ; ++j) drain_part(0, j);
       __builtin_amdgcn_sched_barrier(0);
     }
     const char* xs = lds + x_cur;
@@ -348,8 +371,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
       for (int r = 0; r < 16; ++r)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int m = 4 * r + j;
+        for (int j = 0; j < kJ; ++j) {
+          const int m = kJ * r + j;
           const int g = 16 * half + r;
           if (kDrain != 0 && half == 0) {
             mma16_first(now[2 * j + half], xf[g & 3], acc[r][j]);
@@ -363,7 +386,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
             if (kDrain == 1 && r == 0) drain_store(7, j);
           }
           if (j == 0 && g + 3 < 32) read_frag(g + 3);
-          if ((m & 7) == 2 && m < 32) {
+          if ((m & 7) == 2 && (m >> 3) < kJ) {
             const int j1 = m >> 3;
             if (half == 0) {
               other[2 * j1 + 1] = *reinterpret_cast<const vec8*>(wfrag + (size_t)s_h1 * kBlockBytes + woff[j1] + 1024);
@@ -371,17 +394,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
               now[2 * j1] = *reinterpret_cast<const vec8*>(wfrag + (size_t)s_h0 * kBlockBytes + woff[j1]);
             }
           }
-          if (half == 1 && m >= 6 && (m - 6) % 7 == 0 && m < 6 + 56) {
-            const int i = (m - 6) / 7;
+          constexpr int kDmaFirst = kJ == 4 ? 6 : 4, kDmaEvery = kJ == 4 ? 7 : 5;  // 8 loads over the pass's 16 kJ slots
+          if (half == 1 && m >= kDmaFirst && (m - kDmaFirst) % kDmaEvery == 0 && m < kDmaFirst + 8 * kDmaEvery) {
+            const int i = (m - kDmaFirst) / kDmaEvery;
             dma16(xbytes + (size_t)s_h0 * (BK * 2), xoff[i], fill + 4096u * i);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
     }
     // The x tile of the next step, requested during the previous step, must have landed in every wavefront's
-    // part before anyone reads it: younger than those requests are the 8 weight loads and the 8 direct loads
+    // part before anyone reads it: younger than those requests are the 2 kJ weight loads and the 8 direct loads
     // of this step (stores of a tile's epilogue in between only make the count stricter).
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if constexpr (kJ == 4) {
+      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+    }
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     const int done = x_cur;
@@ -431,8 +459,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int pass = 0; pass < 256 / kStageRows; ++pass) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int cl = 16 * j + 4 * q;  // column inside the wavefront's 64
+      for (int j = 0; j < kJ; ++j) {
+        const int cl = 16 * j + 4 * q;  // column inside the wavefront's 16 kJ
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if constexpr (kBias) {
           const float4 b4 = *reinterpret_cast<const float4*>(bias_f + cl);
@@ -497,6 +525,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           continue;
         }
       }
+      if constexpr (kJ != 4) {  // 6 pieces to a staged row: read-back k takes pieces 64 k + lane in row-major order
+#pragma unroll
+        for (int k = 0; k < kStageRows * 2 * kJ / 64; ++k) {
+          const int idx = 64 * k + lane, rl = idx / (2 * kJ), piece = idx - rl * (2 * kJ);
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + rl * kStageStride + 16 * piece);
+          const int row = m0 + kStageRows * pass + rl, col = n0 + wn + 8 * piece;
+          if (row < M && col < N) *reinterpret_cast<u32x4*>(yout + (int64_t)(row - m0) * out_stride + (col - n0)) = v;
+          if (k & 1) __builtin_amdgcn_sched_barrier(0);
+        }
+        continue;
+      }
 #pragma unroll
       for (int k = 0; k < kStageRows / 8; ++k) {
         const int rl = 8 * k + (lane >> 3);
@@ -526,18 +565,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const char* tb = reinterpret_cast<const char*>(lr_t) + 16 * q;
     const char* bb = reinterpret_cast<const char*>(lr_bs) + 16 * q;
     const uint32_t pitch = (uint32_t)lr_rank * 2u;  // bytes per row of either matrix
-    uint32_t boff[4];
+    uint32_t boff[kJ];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) boff[j] = (uint32_t)min(n0 + wn + 16 * j + c16, N - 1) * pitch;
+    for (int j = 0; j < kJ; ++j) boff[j] = (uint32_t)min(n0 + wn + 16 * j + c16, N - 1) * pitch;
     const uint32_t toff = (uint32_t)min(m0 + c16, M - 1) * pitch;
     const uint32_t t_last = (uint32_t)(M - 1) * pitch;  // rows 16 r + c16 of the tile: 16 * pitch apart until the clamp
     const vec8 zero = __builtin_bit_cast(vec8, make_uint4(0u, 0u, 0u, 0u));
 #pragma unroll 1
     for (uint32_t kb = 0; kb < pitch; kb += 64) {
       const bool in_rank = kb + 16u * (uint32_t)q < pitch;  // a rank of 16 (mod 32) fills half of the last chunk
-      vec8 wf[4];
+      vec8 wf[kJ];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) wf[j] = in_rank ? *reinterpret_cast<const vec8*>(bb + boff[j] + kb) : zero;
+      for (int j = 0; j < kJ; ++j) wf[j] = in_rank ? *reinterpret_cast<const vec8*>(bb + boff[j] + kb) : zero;
 #pragma unroll
       for (int quarter = 0; quarter < 4; ++quarter) {
         vec8 tf[4];
@@ -549,7 +588,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) mma16(wf[j], tf[i], acc[4 * quarter + i][j]);
+          for (int j = 0; j < kJ; ++j) mma16(wf[j], tf[i], acc[4 * quarter + i][j]);
       }
     }
   };
@@ -558,12 +597,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   // between the instructions in front and behind.
   auto settle = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < 16; r += 4)
-      asm volatile("s_nop 15\n\ts_nop 15"
-                   : "+a"(acc[r][0]), "+a"(acc[r][1]), "+a"(acc[r][2]), "+a"(acc[r][3]), "+a"(acc[r + 1][0]),
-                     "+a"(acc[r + 1][1]), "+a"(acc[r + 1][2]), "+a"(acc[r + 1][3]), "+a"(acc[r + 2][0]),
-                     "+a"(acc[r + 2][1]), "+a"(acc[r + 2][2]), "+a"(acc[r + 2][3]), "+a"(acc[r + 3][0]),
-                     "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]), "+a"(acc[r + 3][3]));
+    for (int r = 0; r < 16; r += 4) {
+      if constexpr (kJ == 4) {
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(acc[r][0]), "+a"(acc[r][1]), "+a"(acc[r][2]), "+a"(acc[r][3]), "+a"(acc[r + 1][0]),
+                       "+a"(acc[r + 1][1]), "+a"(acc[r + 1][2]), "+a"(acc[r + 1][3]), "+a"(acc[r + 2][0]),
+                       "+a"(acc[r + 2][1]), "+a"(acc[r + 2][2]), "+a"(acc[r + 2][3]), "+a"(acc[r + 3][0]),
+                       "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]), "+a"(acc[r + 3][3]));
+      } else {
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(acc[r][0]), "+a"(acc[r][1]), "+a"(acc[r][2]), "+a"(acc[r + 1][0]), "+a"(acc[r + 1][1]),
+                       "+a"(acc[r + 1][2]), "+a"(acc[r + 2][0]), "+a"(acc[r + 2][1]), "+a"(acc[r + 2][2]),
+                       "+a"(acc[r + 3][0]), "+a"(acc[r + 3][1]), "+a"(acc[r + 3][2]));
+      }
+    }
   };
 
   // Behind an epilogue: new values for the accumulators (the next item's first step overwrites them anyway), so
@@ -572,7 +619,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int r = 0; r < 16; ++r)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < kJ; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[r][j][e] = 0.f;
   };
@@ -589,6 +636,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     const int q = lane_e >> 4;
     const int lane = lane_e;
     char* stage = lds + kXBuffers * kTileBytes + wave * kStageBytes;
+    if constexpr (kJ == 4) {
 #pragma unroll
     for (int pass = 0; pass < 8; ++pass) {
 #pragma unroll
@@ -608,6 +656,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
         *reinterpret_cast<float4*>(plane + (32 * pass + rl) * BN + wn + 4 * (lane & 15)) = v;
         if (k & 1) __builtin_amdgcn_sched_barrier(0);
       }
+    }
     }
   };
 
@@ -665,7 +714,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       if constexpr (!kPlanes && !kEpi) {
         // A tile with all of its rows and columns inside y and no output bias, followed by another whole
         // tile, leaves its sums in the accumulators: the next tile's first step stores them.
-        if (seq + (int)gridDim.x < end && m0 + BM <= M && n0 + BN <= N && !out_bias) {
+        if (seq + (int)gridDim.x < end && m0 + BM <= M && n0 + kBN <= N && !out_bias) {
           drain_out = out_base;
           pending = true;
           continue;
@@ -717,14 +766,14 @@ int launch_dequant(const uint32_t* wq, const void* scales, const void* biases, i
   return launch_dequant_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
 }
 
-template <typename T, bool kEpi, bool kCut, bool kLowRank>
+template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4>
 int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const void* bias, int64_t N, void* y,
                 int n_whole, int splits, float* planes, hipStream_t stream, LowRank lr, Epilogue epi) {
-  auto kernel = frag_gemm_kernel<T, kEpi, kCut, kLowRank>;
+  auto kernel = frag_gemm_kernel<T, kEpi, kCut, kLowRank, kJ>;
   static PerDeviceInt configured;
   if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
-  const int tiles_n = (int)((N + BN - 1) / BN);
+  const int tiles_n = (int)((N + 64 * kJ - 1) / (64 * kJ));
   const int n_tail = tiles_m * tiles_n - n_whole;
   const int n_items = n_whole + n_tail * splits;
   const int grid = n_items < compute_units() ? n_items : compute_units();  // one persistent workgroup per CU
@@ -750,6 +799,16 @@ int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const 
   };
   const std::true_type yes{};
   const std::false_type no{};
+  // 192-column tiles where they fit one round of workgroups (the 256-column tiles of the same shape then do
+  // too, with a third more work on each of fewer workgroups), unless the plan cuts that round along K
+  const int64_t tiles_192 = ((M + BM - 1) / BM) * ((N + 191) / 192);
+  if (epi.kind == kEpiNone && splits == 1 && tiles_192 <= compute_units()) {
+    if (lr.R)
+      return launch_gemm<T, false, false, true, 3>(x, M, K, workspace, bias, N, y, (int)tiles_192, 1, planes, stream, lr,
+                                                   epi);
+    return launch_gemm<T, false, false, false, 3>(x, M, K, workspace, bias, N, y, (int)tiles_192, 1, planes, stream, lr,
+                                                  epi);
+  }
   if (lr.R) return splits > 1 ? go(no, yes, yes) : go(no, no, yes);  // (no entry point combines update and epilogue)
   if (epi.kind != kEpiNone) return splits > 1 ? go(yes, yes, no) : go(yes, no, no);
   return splits > 1 ? go(no, yes, no) : go(no, no, no);

@@ -39,10 +39,12 @@ def _call(lib, name, code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y, ws, ws_b
 
 # 17 x 13 tiles = 221 of 256 CUs: the shape class the path takes; M and N ragged (N % 16 == 8)
 # K = 512: four blocks of 64 k per wavefront and trip of the copy kernel; K = 384 and 640: two
+# M = 2400: 10 x 17 tiles of 192 columns fit the 256 CUs, which is when the path uses those
+@pytest.mark.parametrize("M", [4100, 2400])
 @pytest.mark.parametrize("bits,gs,dtype,with_bias,K", [
     (4, 64, "bf16", True, 512), (8, 64, "bf16", False, 512), (4, 32, "bf16", False, 512), (8, 128, "bf16", True, 512),
     (4, 128, "f16", True, 512), (8, 32, "f16", False, 512), (4, 64, "bf16", False, 640), (8, 64, "f16", True, 384)])
-def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_bias, K):
+def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_bias, K, M):
     from gpu_util import to_dev, u32_to_dev
     from mflux_amd import _lib
 
@@ -50,7 +52,7 @@ def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_
     lib = _lib.load()
     dt = o.BF16 if dtype == "bf16" else o.F16
     code = _lib.BF16 if dtype == "bf16" else _lib.F16
-    M, N = 4100, 3208
+    N = 3208
     need = lib.mfq_qmm_t_workspace_bytes(M, K, N, gs, bits)
     n16 = (N + 15) // 16 * 16
     assert need == n16 * K * 2, "the shape must take the two-kernel path, uncut"
