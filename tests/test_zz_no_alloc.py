@@ -42,8 +42,10 @@ def test_static_scratch_matches_workspace_call_twice(oracle):
     lib = _lib.load()
     # (M, K, N, bits): a text-stream shape the 128-column kernel cuts along K, then a smaller one that is cut too;
     # the third call has 256 x 256 tiles whose short last round is cut (the fused large-M kernel's planes); the
-    # fourth runs the two-kernel path with its 16-bit copy of the weights in the buffer
-    shapes = [(512, 3072, 3072, 4), (300, 2048, 1024, 8), (2040, 3072, 8448, 4), (4608, 512, 3072, 4)]
+    # fourth runs the two-kernel path with its 16-bit copy of the weights in the buffer, the fifth too, on
+    # 192-column tiles (ragged in M and N)
+    shapes = [(512, 3072, 3072, 4), (300, 2048, 1024, 8), (2040, 3072, 8448, 4), (4608, 512, 3072, 4),
+              (2400, 512, 3208, 8)]
     for idx, (M, K, N, bits) in enumerate(shapes):
         need = lib.mfq_qmm_t_workspace_bytes(M, K, N, 64, bits)
         assert 0 < need <= STATIC_BYTES, f"case {idx} must exercise the scratch buffer (needs {need} bytes)"
