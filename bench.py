@@ -371,6 +371,20 @@ def main():
         library[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
         del w16
 
+    # ---- secondary: the same linears on a prepared copy of their weights -------
+    # (the 16-bit copy made once instead of on every call, 2 bytes per weight held: the GEMM kernel alone)
+    prepared = {}
+    for name, x, wq, s, b in (() if args.no_secondary else ops):
+        K, N = x.shape[1], wq.shape[0]
+        copy = mflux_amd.prepare_weights(wq, s, b, group_size=GS, bits=BITS)
+        for _ in range(3):
+            mflux_amd.quantized_matmul_prepared(x, copy, N)
+        torch.cuda.synchronize()
+        ms = event_ms(lambda: mflux_amd.quantized_matmul_prepared(x, copy, N), 20, torch)
+        prepared[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1),
+                          "copy_mb_held": round(copy.numel() / 1e6, 1)}
+        del copy
+
     # ---- secondary: a rank-16 LoRA on the two linears --------------------------
     # the whole layer (x @ A included) as one fused call against the reference's
     # composition of separate matmuls, and the kernel alone with the update
@@ -579,7 +593,7 @@ def main():
                       "gemv_w8": gemv.get("w8", {}),
                       "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
                       "qmm_w4_lora_r16": lora, "epilogues_fused_vs_separate": fused,
-                      "library_bf16_gemm_same_operands": library},
+                      "library_bf16_gemm_same_operands": library, "qmm_w4_prepared_weights": prepared},
     }
     if not args.no_cpu_baseline:
         name, x, wq, s, b = ops[0]

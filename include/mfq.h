@@ -236,6 +236,33 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
                  size_t workspace_bytes, void* stream);
 
 /*
+ * The two halves of a large mfq_qmm_t_ws call apart, for weights that do not
+ * change between calls (inference).  Has no counterpart in the reference: MLX
+ * dequantises inside every quantized_matmul.  mfq_qmm_t_prepare writes the
+ * 16-bit copy of the dequantised weights that mfq_qmm_t_ws makes per call --
+ * one rounding of fma(code, scale, bias) to sb_dtype, in the order the matrix
+ * instructions consume it, mfq_qmm_t_prepared_bytes(N, K, bits) bytes (2 per
+ * weight; 0: no such copy for this shape: bits other than 4 or 8, K not a
+ * multiple of 128 or below 256, N not a multiple of 8, or more than 2 GiB) --
+ * into a buffer the caller keeps, and mfq_qmm_t_prepared multiplies x
+ * [M, K] of the same 16-bit type with it into y [M, N] of that type (+ bias):
+ * bit-identical to what mfq_qmm_t_ws gives on its two-kernel path, for any M,
+ * at 2 bytes per weight of memory held instead of bits / 8 -- on FLUX.1's
+ * single-block linears at M = 4608 the copy is 7 % of the call.  The copy can
+ * also be made on another stream while the previous layer's product runs.
+ * `workspace` (optional, 16-byte aligned, mfq_qmm_t_prepared_workspace_bytes)
+ * takes the float32 planes of a K cut of a short last round of tiles; without
+ * it the tiles run whole.  MFQ_EUNSUPPORTED for shapes without a copy.
+ */
+size_t mfq_qmm_t_prepared_bytes(int64_t N, int64_t K, int bits);
+int mfq_qmm_t_prepare(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype,
+                      int64_t N, int64_t K, int group_size, int bits, void* prepared, void* stream);
+size_t mfq_qmm_t_prepared_workspace_bytes(int64_t M, int64_t K, int64_t N);
+int mfq_qmm_t_prepared(const void* x, int dtype, int64_t M, int64_t K, const void* prepared,
+                       const void* bias, int64_t N, void* y, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/*
  * mfq_qmm_t_ws for callers that cannot allocate: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  Has no counterpart in
  * the reference.  The float32 planes of the K split live in a buffer of

@@ -31,6 +31,10 @@ SIGNATURES = {
     "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,
                             ctypes.c_size_t, _PTR]),
+    "mfq_qmm_t_prepared_bytes": (ctypes.c_size_t, [_I64, _I64, _INT]),
+    "mfq_qmm_t_prepare": (_INT, [_PTR, _PTR, _PTR, _INT, _I64, _I64, _INT, _INT, _PTR, _PTR]),
+    "mfq_qmm_t_prepared_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64]),
+    "mfq_qmm_t_prepared": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _I64, _PTR, _PTR, ctypes.c_size_t, _PTR]),
     "mfq_qmm_t_static": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_qmm_t_low_rank": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _PTR,
                                   _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),

@@ -240,6 +240,75 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
 
 
 
+def prepare_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64,
+                    bits: int = 4) -> torch.Tensor | None:
+    """The 16-bit copy of ``dequantize(w)`` that a large ``quantized_matmul``
+    makes on every call, made once: for weights that do not change between calls
+    and a caller with 2 bytes per weight of device memory to spare
+    (``include/mfq.h``: ``mfq_qmm_t_prepare``).  Not part of MLX, which
+    dequantises inside every ``mx.quantized_matmul``.  Returns an opaque uint8
+    tensor for ``quantized_matmul_prepared``, or ``None`` where the library has
+    no such copy for the shape (bits other than 4 or 8, ``K`` not a multiple of
+    128, ``N`` not a multiple of 8).  The values are those every other kernel
+    multiplies with: one rounding of ``fma(code, scale, bias)`` to the dtype of
+    ``scales``."""
+    _check_group_bits("prepare_weights", group_size, bits)
+    _check_packed("prepare_weights", w, scales, biases, group_size, bits)
+    if w.ndim != 2 or scales.dtype not in (torch.float16, torch.bfloat16):
+        return None
+    _require_hip("prepare_weights", w, "w")
+    lib = _lib.load()
+    N, K = w.shape[0], w.shape[1] * 32 // bits
+    need = lib.mfq_qmm_t_prepared_bytes(N, K, bits)
+    if need == 0:
+        return None
+    w, scales, biases = w.contiguous(), scales.contiguous(), biases.contiguous()
+    out = torch.empty(need, dtype=torch.uint8, device=w.device)
+    with torch.cuda.device(w.device):
+        rc = lib.mfq_qmm_t_prepare(w.data_ptr(), scales.data_ptr(), biases.data_ptr(), _DTYPE_CODE[scales.dtype], N, K,
+                                   group_size, bits, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise _lib.MfqError("mfq_qmm_t_prepare", rc, lib.mfq_strerror(rc).decode())
+    return out
+
+
+def quantized_matmul_prepared(x: torch.Tensor, prepared: torch.Tensor, output_dims: int,
+                              bias: torch.Tensor | None = None) -> torch.Tensor:
+    """``x @ dequantize(w).T (+ bias)`` on the copy ``prepare_weights`` made of
+    ``w``: the second kernel of a large ``quantized_matmul`` alone, with the same
+    bits in its result.  ``x``: ``[..., K]`` of the 16-bit dtype the copy was
+    made in (the dtype of the scales); any number of rows, meant for some
+    thousands (below that ``quantized_matmul``'s other kernels are the faster
+    ones).  Inference only."""
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"[quantized_matmul_prepared] x must be float16 or bfloat16, got {x.dtype}")
+    _require_hip("quantized_matmul_prepared", x, "x")
+    lib = _lib.load()
+    N, K = int(output_dims), x.shape[-1]
+    if prepared.dtype != torch.uint8 or prepared.numel() != lib.mfq_qmm_t_prepared_bytes(N, K, 4):
+        raise ValueError(f"[quantized_matmul_prepared] the prepared copy does not belong to a weight of {N} x {K}")
+    lead = tuple(x.shape[:-1])
+    x2 = x.reshape(-1, K).contiguous()
+    M = x2.shape[0]
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    if M == 0:
+        return y.reshape(*lead, N)
+    if bias is not None:
+        if bias.shape != (N,):
+            raise ValueError(f"[quantized_matmul_prepared] bias must have shape ({N},), got {tuple(bias.shape)}")
+        bias = bias.to(x.dtype).contiguous()
+    ws_bytes = lib.mfq_qmm_t_prepared_workspace_bytes(M, K, N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    with torch.cuda.device(x.device):
+        rc = lib.mfq_qmm_t_prepared(x2.data_ptr(), _DTYPE_CODE[x.dtype], M, K, prepared.data_ptr(),
+                                    None if bias is None else bias.data_ptr(), N, y.data_ptr(),
+                                    None if ws is None else ws.data_ptr(), ws_bytes,
+                                    torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise _lib.MfqError("mfq_qmm_t_prepared", rc, lib.mfq_strerror(rc).decode())
+    return y.reshape(*lead, N)
+
+
 def silu(x: torch.Tensor) -> torch.Tensor:
     """``x * sigmoid(x)`` as MLX's ``nn.silu`` evaluates it: two operations in
     ``x``'s dtype, so on a 16-bit tensor the sigmoid is rounded before the

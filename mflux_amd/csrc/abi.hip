@@ -129,6 +129,37 @@ int mfq_qmm_t_static(const void* x, int x_dtype, int64_t M, int64_t K, const uin
                             0, y, y_dtype, ws, need, stream);
 }
 
+size_t mfq_qmm_t_prepared_bytes(int64_t N, int64_t K, int bits) {
+  if (N <= 0 || K <= 0 || N > INT32_MAX || K > INT32_MAX || !mfq::qmm_frag_shape_ok(1, N, K, bits)) return 0;
+  return mfq::qmm_frag_copy_bytes(N, K);
+}
+
+int mfq_qmm_t_prepare(const uint32_t* wq, const void* scales, const void* biases, int sb_dtype, int64_t N, int64_t K,
+                      int group_size, int bits, void* prepared, void* stream) {
+  if (int rc = check_common(group_size, bits)) return rc;
+  if (!is16(sb_dtype)) return MFQ_EDTYPE;
+  if (N <= 0 || K <= 0 || K % group_size || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!wq || !scales || !biases || !prepared) return MFQ_ENULL;
+  if (!mfq::aligned16(wq) || !mfq::aligned16(prepared)) return MFQ_EALIGN;
+  return mfq::launch_qmm_frag_copy(sb_dtype, wq, scales, biases, N, K, group_size, bits, prepared, (hipStream_t)stream);
+}
+
+size_t mfq_qmm_t_prepared_workspace_bytes(int64_t M, int64_t K, int64_t N) {
+  if (M <= 0 || N <= 0 || K <= 0 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  if (!mfq::qmm_frag_shape_ok(M, N, K, 4)) return 0;
+  return mfq::qmm_prepared_workspace_bytes(M, N, K);
+}
+
+int mfq_qmm_t_prepared(const void* x, int dtype, int64_t M, int64_t K, const void* prepared, const void* bias, int64_t N,
+                       void* y, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!is16(dtype)) return MFQ_EDTYPE;
+  if (M <= 0 || N <= 0 || K <= 0) return MFQ_ESHAPE;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return MFQ_ESHAPE;
+  if (!x || !prepared || !y) return MFQ_ENULL;
+  if (!mfq::aligned16(x) || !mfq::aligned16(prepared) || !mfq::aligned16(y)) return MFQ_EALIGN;
+  return mfq::launch_qmm_prepared(x, dtype, M, K, prepared, bias, N, y, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                        const void* biases, int sb_dtype, const void* bias, int64_t N, int group_size, int bits,
                        const void* t, const void* bs, int64_t rank, void* y, int y_dtype, void* workspace,

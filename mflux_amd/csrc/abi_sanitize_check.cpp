@@ -97,6 +97,17 @@ int main() {
          MFQ_ESHAPE);
   if (mfq_qmm_t_workspace_bytes(0, 128, 8, 64, 4) != 0 || mfq_qmm_t_workspace_bytes(4, 100, 8, 64, 4) != 0) ++failures;
 
+  expect("prepare: dtype", mfq_qmm_t_prepare(u, p, p, MFQ_F32, 64, 256, 64, 4, p, nullptr), MFQ_EDTYPE);
+  expect("prepare: K", mfq_qmm_t_prepare(u, p, p, MFQ_BF16, 64, 250, 64, 4, p, nullptr), MFQ_ESHAPE);
+  expect("prepare: null", mfq_qmm_t_prepare(u, p, nullptr, MFQ_BF16, 64, 256, 64, 4, p, nullptr), MFQ_ENULL);
+  expect("prepare: bits", mfq_qmm_t_prepare(u, p, p, MFQ_BF16, 64, 256, 64, 6, p, nullptr), MFQ_EUNSUPPORTED);
+  expect("prepared: dtype", mfq_qmm_t_prepared(p, MFQ_F32, 4, 256, p, nullptr, 64, p, nullptr, 0, nullptr), MFQ_EDTYPE);
+  expect("prepared: M", mfq_qmm_t_prepared(p, MFQ_BF16, 0, 256, p, nullptr, 64, p, nullptr, 0, nullptr), MFQ_ESHAPE);
+  expect("prepared: null", mfq_qmm_t_prepared(p, MFQ_BF16, 4, 256, nullptr, nullptr, 64, p, nullptr, 0, nullptr), MFQ_ENULL);
+  expect("prepared: K", mfq_qmm_t_prepared(p, MFQ_BF16, 4, 192, p, nullptr, 64, p, nullptr, 0, nullptr), MFQ_EUNSUPPORTED);
+  if (mfq_qmm_t_prepared_bytes(64, 192, 4) != 0 || mfq_qmm_t_prepared_bytes(64, 256, 4) != 64 * 256 * 2) ++failures;
+  if (mfq_qmm_t_prepared_workspace_bytes(0, 256, 64) != 0) ++failures;
+
   std::free(raw);
   if (failures) return 1;
   std::printf("abi_sanitize_check: every refusal clean\n");

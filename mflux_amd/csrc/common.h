@@ -360,6 +360,17 @@ size_t qmm_frag_copy_bytes(int64_t N, int64_t K);
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
                     int n_whole, int splits, hipStream_t stream, LowRank low_rank, Epilogue epi);
+// its two halves apart: the copy alone (weights that do not change between calls need it once), and the GEMM on a
+// copy made before, with the planes of a K cut wherever the caller has room for them
+int launch_qmm_frag_copy(int dtype, const uint32_t* wq, const void* scales, const void* biases, int64_t N, int64_t K,
+                         int gs, int bits, void* copy, hipStream_t stream);
+int launch_qmm_frag_gemm(const void* x, int dtype, int64_t M, int64_t K, const void* copy, const void* bias, int64_t N,
+                         void* y, float* planes, int n_whole, int splits, hipStream_t stream, LowRank low_rank,
+                         Epilogue epi);
+// the GEMM on a prepared copy with the K cut planned here: `workspace` takes the planes (without room: whole tiles)
+size_t qmm_prepared_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int launch_qmm_prepared(const void* x, int dtype, int64_t M, int64_t K, const void* copy, const void* bias, int64_t N,
+                        void* y, void* workspace, size_t workspace_bytes, hipStream_t stream);
 // y tiles = sums of the planes of a K cut (+ bias, epilogue): the second kernel of qmm.hip's and qmm_frag.hip's cut
 int launch_tail_reduce(int dtype, const float* planes, int n_whole, int splits, int tiles_m, int tiles_n,
                        const void* bias, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream, Epilogue epi);

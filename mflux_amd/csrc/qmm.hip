@@ -1169,6 +1169,23 @@ int launch_splitk_reduce(int dtype, const void* planes, int splits, int64_t M, i
   return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
 }
 
+// The K cut of the two-kernel path's GEMM when the copy is already there: ranges of whole pairs of k steps.
+size_t qmm_prepared_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (K % (2 * BK)) return 0;
+  return tail_plane_bytes(M, N, plan_tail(M, N, K, 2, compute_units()));
+}
+
+int launch_qmm_prepared(const void* x, int dtype, int64_t M, int64_t K, const void* copy, const void* bias, int64_t N,
+                        void* y, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  if (!qmm_frag_shape_ok(M, N, K, 4)) return MFQ_EUNSUPPORTED;
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  TailPlan plan = plan_tail(M, N, K, 2, compute_units());
+  if (plan.splits > 1 && (!workspace || !aligned16(workspace) || workspace_bytes < tail_plane_bytes(M, N, plan)))
+    plan = TailPlan{(int)tiles, 1};
+  return launch_qmm_frag_gemm(x, dtype, M, K, copy, bias, N, y, static_cast<float*>(workspace), plan.n_whole,
+                              plan.splits, stream, LowRank(), Epilogue());
+}
+
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank, Epilogue epi) {

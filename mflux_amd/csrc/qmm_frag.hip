@@ -787,15 +787,11 @@ int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const vo
 }
 
 template <typename T>
-int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const void* scales, const void* biases,
-                 const void* bias, int64_t N, int gs, int bits, void* y, void* workspace, int n_whole, int splits,
-                 hipStream_t stream, LowRank lr, Epilogue epi) {
-  if (int rc = launch_dequant<T>(wq, scales, biases, gs, bits, workspace, N, K, stream)) return rc;
-  // the planes of a K cut lie behind the copy
-  float* planes = reinterpret_cast<float*>(static_cast<char*>(workspace) + qmm_frag_copy_bytes(N, K));
+int launch_gemm_typed(const void* x, int64_t M, int64_t K, const void* copy, const void* bias, int64_t N, void* y,
+                      float* planes, int n_whole, int splits, hipStream_t stream, LowRank lr, Epilogue epi) {
   auto go = [&](auto e, auto c, auto l) {
     return launch_gemm<T, decltype(e)::value, decltype(c)::value, decltype(l)::value>(
-        x, M, K, workspace, bias, N, y, n_whole, splits, planes, stream, lr, epi);
+        x, M, K, copy, bias, N, y, n_whole, splits, planes, stream, lr, epi);
   };
   const std::true_type yes{};
   const std::false_type no{};
@@ -804,10 +800,8 @@ int launch_typed(const void* x, int64_t M, int64_t K, const uint32_t* wq, const 
   const int64_t tiles_192 = ((M + BM - 1) / BM) * ((N + 191) / 192);
   if (epi.kind == kEpiNone && splits == 1 && tiles_192 <= compute_units()) {
     if (lr.R)
-      return launch_gemm<T, false, false, true, 3>(x, M, K, workspace, bias, N, y, (int)tiles_192, 1, planes, stream, lr,
-                                                   epi);
-    return launch_gemm<T, false, false, false, 3>(x, M, K, workspace, bias, N, y, (int)tiles_192, 1, planes, stream, lr,
-                                                  epi);
+      return launch_gemm<T, false, false, true, 3>(x, M, K, copy, bias, N, y, (int)tiles_192, 1, planes, stream, lr, epi);
+    return launch_gemm<T, false, false, false, 3>(x, M, K, copy, bias, N, y, (int)tiles_192, 1, planes, stream, lr, epi);
   }
   if (lr.R) return splits > 1 ? go(no, yes, yes) : go(no, no, yes);  // (no entry point combines update and epilogue)
   if (epi.kind != kEpiNone) return splits > 1 ? go(yes, yes, no) : go(yes, no, no);
@@ -826,21 +820,37 @@ bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits) {
 // the copy, rounded up to whole 256 bytes so that what lies behind it is aligned
 size_t qmm_frag_copy_bytes(int64_t N, int64_t K) { return ((size_t)(((N + 15) / 16) * 16 * K * 2) + 255) & ~(size_t)255; }
 
-int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
-                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
-                    int n_whole, int splits, hipStream_t stream, LowRank lr, Epilogue epi) {
-  if (!qmm_frag_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+int launch_qmm_frag_copy(int dtype, const uint32_t* wq, const void* scales, const void* biases, int64_t N, int64_t K,
+                         int gs, int bits, void* copy, hipStream_t stream) {
+  if (!qmm_frag_shape_ok(1, N, K, bits)) return MFQ_EUNSUPPORTED;
+  if (dtype == MFQ_BF16) return launch_dequant<BF16>(wq, scales, biases, gs, bits, copy, N, K, stream);
+  if (dtype == MFQ_F16) return launch_dequant<F16>(wq, scales, biases, gs, bits, copy, N, K, stream);
+  return MFQ_EDTYPE;
+}
+
+int launch_qmm_frag_gemm(const void* x, int dtype, int64_t M, int64_t K, const void* copy, const void* bias, int64_t N,
+                         void* y, float* planes, int n_whole, int splits, hipStream_t stream, LowRank lr,
+                         Epilogue epi) {
+  if (!qmm_frag_shape_ok(M, N, K, 4)) return MFQ_EUNSUPPORTED;
   if (lr.R && (epi.kind != kEpiNone || lr.R % 16)) return MFQ_EUNSUPPORTED;
   // 32-bit byte offsets into the update's operands
   if ((M + BM) * lr.R >= (int64_t)1 << 31 || (N + BN) * lr.R >= (int64_t)1 << 31) return MFQ_EUNSUPPORTED;
   if (splits > 1 && ((K / BK) % splits || (K / BK / splits) % 2)) return MFQ_EUNSUPPORTED;  // ranges of whole pairs of steps
   if (dtype == MFQ_BF16)
-    return launch_typed<BF16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, lr,
-                              epi);
+    return launch_gemm_typed<BF16>(x, M, K, copy, bias, N, y, planes, n_whole, splits, stream, lr, epi);
   if (dtype == MFQ_F16)
-    return launch_typed<F16>(x, M, K, wq, scales, biases, bias, N, gs, bits, y, workspace, n_whole, splits, stream, lr,
-                             epi);
+    return launch_gemm_typed<F16>(x, M, K, copy, bias, N, y, planes, n_whole, splits, stream, lr, epi);
   return MFQ_EDTYPE;
+}
+
+int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
+                    int n_whole, int splits, hipStream_t stream, LowRank lr, Epilogue epi) {
+  if (!qmm_frag_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+  if (int rc = launch_qmm_frag_copy(dtype, wq, scales, biases, N, K, gs, bits, workspace, stream)) return rc;
+  // the planes of a K cut lie behind the copy
+  float* planes = reinterpret_cast<float*>(static_cast<char*>(workspace) + qmm_frag_copy_bytes(N, K));
+  return launch_qmm_frag_gemm(x, dtype, M, K, workspace, bias, N, y, planes, n_whole, splits, stream, lr, epi);
 }
 
 }  // namespace mfq

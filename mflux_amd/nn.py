@@ -94,7 +94,30 @@ class QuantizedLinear(torch.nn.Module):
         return (f"input_dims={self.input_dims}, output_dims={self.output_dims}, bias={self.bias is not None}, "
                 f"group_size={self.group_size}, bits={self.bits}, mode={self.mode}")
 
+    PREPARED_MIN_ROWS = 2048  # from here on forward() multiplies with the prepared copy, if there is one
+
+    def _weights_key(self):
+        return tuple((t.data_ptr(), t._version) for t in (self.weight, self.scales, self.biases))
+
+    def prepare(self) -> bool:
+        """Keeps a 16-bit copy of the dequantised weights in the order the large-M
+        GEMM consumes them (``core.prepare_weights``: 2 bytes per weight of device
+        memory), so that calls with thousands of rows skip the dequantisation
+        pass.  Not part of MLX's layer.  The copy is not part of ``state_dict()``
+        and is made again when the layer's tensors have been replaced or written
+        to.  Returns False (and keeps nothing) where the library has no such copy
+        for the layer's shape."""
+        self._prepared = core.prepare_weights(self.weight, self.scales, self.biases, self.group_size, self.bits)
+        self._prepared_key = self._weights_key() if self._prepared is not None else None
+        return self._prepared is not None
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if (getattr(self, "_prepared", None) is not None and x.dtype == self.scales.dtype and x.shape[-1] > 0
+                and x.numel() // x.shape[-1] >= self.PREPARED_MIN_ROWS and not (torch.is_grad_enabled() and x.requires_grad)):
+            if self._prepared_key != self._weights_key():
+                self.prepare()
+            if self._prepared is not None:
+                return core.quantized_matmul_prepared(x, self._prepared, self.output_dims, self.bias)
         return core.quantized_matmul(x, self.weight, self.scales, self.biases, transpose=True,
                                      group_size=self.group_size, bits=self.bits, mode=self.mode, bias=self.bias)
 

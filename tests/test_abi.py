@@ -21,6 +21,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
                  "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add",
+                 "mfq_qmm_t_prepare", "mfq_qmm_t_prepared", "mfq_qmm_t_prepared_bytes", "mfq_qmm_t_prepared_workspace_bytes",
                  "mfq_qmv_silu"):
         assert must in names
 
@@ -132,6 +133,24 @@ def test_argument_validation_needs_no_device():
     assert add(base, base, _lib.BF16, 4, 8, 24, base, _lib.BF16, None) == E["shape"]
     assert add(base, None, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["null"]
     assert add(base + 8, base, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["align"]
+    # the two halves of the large-M call apart: which shapes have a prepared copy, and the checks of both calls
+    nbytes = lib.mfq_qmm_t_prepared_bytes
+    assert nbytes(3072, 3072, 4) == 3072 * 3072 * 2 and nbytes(3208, 512, 8) == 3216 * 512 * 2
+    assert nbytes(3072, 3072, 5) == 0 and nbytes(3072, 192, 4) == 0 and nbytes(3076, 512, 4) == 0 and nbytes(0, 512, 4) == 0
+    prep = lib.mfq_qmm_t_prepare
+    assert prep(base, base, base, _lib.F32, 64, 256, 64, 4, base, None) == E["dtype"]
+    assert prep(base, base, base, _lib.BF16, 64, 256, 48, 4, base, None) == E["group"]
+    assert prep(base, base, base, _lib.BF16, 64, 250, 64, 4, base, None) == E["shape"]
+    assert prep(base, base, None, _lib.BF16, 64, 256, 64, 4, base, None) == E["null"]
+    assert prep(base, base, base, _lib.BF16, 64, 256, 64, 4, base + 8, None) == E["align"]
+    assert prep(base, base, base, _lib.BF16, 64, 256, 64, 6, base, None) == E["unsupported"]
+    prepared = lib.mfq_qmm_t_prepared
+    assert prepared(base, _lib.F32, 4, 256, base, None, 64, base, None, 0, None) == E["dtype"]
+    assert prepared(base, _lib.BF16, 0, 256, base, None, 64, base, None, 0, None) == E["shape"]
+    assert prepared(base, _lib.BF16, 4, 256, None, None, 64, base, None, 0, None) == E["null"]
+    assert prepared(base, _lib.BF16, 4, 256, base, None, 64, base + 4, None, 0, None) == E["align"]
+    assert prepared(base, _lib.BF16, 4, 192, base, None, 64, base, None, 0, None) == E["unsupported"]
+    assert lib.mfq_qmm_t_prepared_workspace_bytes(4, 192, 64) == 0
     # the matvec with the activation inside: one row of 16-bit x, 4 or 8 bits, rows the one-row kernel takes
     silu = lib.mfq_qmv_silu
 

@@ -255,3 +255,75 @@ def test_two_kernel_path_is_reproducible_bit_for_bit():
                 again = fn()
                 assert torch.equal(first, again), (M, K, N, bits, rank, fn.__name__, i)
         assert bool(torch.isfinite(first).all())
+
+
+@pytest.mark.parametrize("bits,dtype,M,K,N,with_bias", [
+    (4, "bf16", 4608, 256, 7680, False),   # 540 tiles: deferred stores, a K cut of the last 28
+    (8, "f16", 2400, 512, 3208, True),     # 192-column tiles, ragged
+    (4, "bf16", 300, 1024, 2304, True),    # few rows: the same kernel on tiles the other paths would not give it
+])
+def test_prepared_copy_gives_the_two_kernel_paths_bits(oracle, bits, dtype, M, K, N, with_bias):
+    """mfq_qmm_t_prepare + mfq_qmm_t_prepared are the two kernels of a large
+    mfq_qmm_t_ws call apart: the copy is the same bytes, the product the same
+    bits (first two shapes, which mfq_qmm_t_ws runs on that path), and the
+    float64 oracle bounds it for any M."""
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    x, wq, s, b, bias = _operands(o, 160 + bits, M, K, N, bits, 64, dt, with_bias)
+    xd, wd, sd, bd = to_dev(x, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt)
+    biasd = None if bias is None else to_dev(bias, dt)
+    stream = torch.cuda.current_stream().cuda_stream
+    nbytes = lib.mfq_qmm_t_prepared_bytes(N, K, bits)
+    assert nbytes == (N + 15) // 16 * 16 * K * 2
+    copy = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+    assert lib.mfq_qmm_t_prepare(wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), code, N, K, 64, bits, copy.data_ptr(),
+                                 stream) == 0
+    ws_bytes = lib.mfq_qmm_t_prepared_workspace_bytes(M, K, N)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+    y = torch.full((M, N), float("nan"), dtype=xd.dtype, device="cuda")
+    assert lib.mfq_qmm_t_prepared(xd.data_ptr(), code, M, K, copy.data_ptr(),
+                                  None if biasd is None else biasd.data_ptr(), N, y.data_ptr(), ws.data_ptr(),
+                                  ws_bytes, stream) == 0
+    torch.cuda.synchronize()
+    ref = o.quantized_matmul_f64(_to_f64(o, x, dt), wq, s, b, dt, 64, bits,
+                                 bias_f64=None if bias is None else _to_f64(o, bias, dt))
+    err = np.abs(y.double().cpu().numpy() - ref) / np.abs(ref).max(axis=-1, keepdims=True)
+    assert err.max() <= TOL, err.max()
+    need = lib.mfq_qmm_t_workspace_bytes(M, K, N, 64, bits)
+    if need >= nbytes and M >= 2048:
+        full = torch.empty(need, dtype=torch.uint8, device="cuda")
+        y_ws = torch.empty_like(y)
+        assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, 64, bits, xd, wd, sd, bd, biasd, y_ws, full, need) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(full[:nbytes], copy)
+        assert torch.equal(y_ws.view(torch.int16), y.view(torch.int16))
+
+
+def test_quantized_linear_prepare():
+    """QuantizedLinear.prepare(): same bits as the layer gives without it from
+    2048 rows on, the ordinary kernels below that, and a new copy after the
+    layer's tensors have been written to."""
+    import mflux_amd
+
+    torch.manual_seed(5)
+    lin = mflux_amd.nn.QuantizedLinear(512, 3072, bias=True, group_size=64, bits=4, device="cuda")
+    lin.bias.normal_(0, 0.02)
+    x = torch.randn(2, 2304, 512, device="cuda", dtype=torch.bfloat16)
+    small = torch.randn(7, 512, device="cuda", dtype=torch.bfloat16)
+    y0, s0 = lin(x), lin(small)
+    assert lin.prepare()
+    assert "_prepared" not in lin.state_dict()
+    assert torch.equal(lin(x), y0) and torch.equal(lin(small), s0)
+    w2, sc2, b2 = mflux_amd.quantize(torch.randn(3072, 512, device="cuda", dtype=torch.bfloat16) * 0.05, 64, 4)
+    lin.weight.copy_(w2), lin.scales.copy_(sc2), lin.biases.copy_(b2)
+    y1 = mflux_amd.quantized_matmul(x, w2, sc2, b2, bias=lin.bias)
+    assert not torch.equal(y1, y0)
+    assert torch.equal(lin(x), y1)
+    odd = mflux_amd.nn.QuantizedLinear(512, 3072, bias=False, group_size=64, bits=6, device="cuda")
+    assert not odd.prepare()
+    assert odd(x).shape == (2, 2304, 3072)
