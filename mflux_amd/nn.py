@@ -324,6 +324,19 @@ def concat_quantized(layers: list[QuantizedLinear], share_storage: bool = False)
     return out
 
 
+def prepare(model: torch.nn.Module, min_output_dims: int = 0) -> int:
+    """Calls ``QuantizedLinear.prepare()`` on every quantized linear of ``model``
+    with at least ``min_output_dims`` output features (after loading, baking
+    and stacking: the copy follows later changes to a layer's tensors, at the
+    price of making it again).  Not part of MLX.  Returns the bytes of device
+    memory the kept copies take: 2 per weight, 24 GB for FLUX.1's transformer."""
+    held = 0
+    for module in model.modules():
+        if isinstance(module, QuantizedLinear) and module.output_dims >= min_output_dims and module.prepare():
+            held += module._prepared.numel()
+    return held
+
+
 class Linear(torch.nn.Linear):
     """``torch.nn.Linear`` with MLX's ``to_quantized`` hook, so that the
     reference's ``hasattr(module, "to_quantized")`` predicates select it."""

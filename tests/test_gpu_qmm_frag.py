@@ -327,3 +327,8 @@ def test_quantized_linear_prepare():
     odd = mflux_amd.nn.QuantizedLinear(512, 3072, bias=False, group_size=64, bits=6, device="cuda")
     assert not odd.prepare()
     assert odd(x).shape == (2, 2304, 3072)
+    # the walk over a model: every quantized linear that has such a copy, and what they hold together
+    model = torch.nn.Sequential(mflux_amd.nn.QuantizedLinear(512, 1024, device="cuda"), torch.nn.GELU(),
+                                mflux_amd.nn.QuantizedLinear(1024, 512, bits=8, device="cuda"), odd)
+    assert mflux_amd.nn.prepare(model) == 2 * (1024 * 512 + 512 * 1024)
+    assert mflux_amd.nn.prepare(model, min_output_dims=1024) == 2 * 1024 * 512
