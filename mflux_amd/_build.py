@@ -87,7 +87,7 @@ def check_generated_code(src: str) -> int:
     for m in re.finditer(r"^(\S*%s\S*):" % re.escape(ASM_MFMA_KERNELS[src]), text, re.M):
         body = text[m.end():text.index(".Lfunc_end", m.end())]
         n_matrix = 0
-        col_tiles = re.search(r"ELi(\d)EEEv", m.group(1))  # the kernel's last template argument: column tiles per wavefront
+        col_tiles = re.search(r"ELi(\d)ELb[01]EEEv", m.group(1))  # the template argument before the last: column tiles per wavefront
         least = 2 * int(col_tiles.group(1)) if col_tiles else 8
         for block in re.split(r"\n\.LBB[0-9_]+:", body):
             ops = [ln.split()[0] for ln in block.split("\n") if ln.strip() and not ln.strip().startswith((";", "."))]

@@ -182,7 +182,9 @@ __device__ __forceinline__ void acc_read(f32x4& c, float (&v)[4]) {
 // kJ: column tiles of 16 per wavefront, i.e. tiles of 256 rows x 64 kJ columns: 4, or 3 (192 columns) for
 //     shapes whose 192-column tiles fit one round of workgroups (a quarter less work per workgroup than the
 //     256-column tiles of the same round); without epilogue or K cut
-template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4>
+// kDeferBias: the instantiation for calls with an output bias, whose deferred tile stores (do_step) add it
+//     (apart, because the add in the slots of the other costs the calls without a bias a fifth of that pass)
+template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4, bool kDeferBias = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void frag_gemm_kernel(
     const uint16_t* __restrict__ x, const char* __restrict__ wfrag, const uint16_t* __restrict__ bias,
     void* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n, int n_whole, int tail_splits,
@@ -191,6 +193,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
   extern __shared__ __attribute__((aligned(16))) char lds[];
   using vec8 = typename T::vec8;
   static_assert(kJ == 4 || (kJ == 3 && !kEpi && !kCut), "192-column tiles: plain whole tiles only");
+  static_assert(!kDeferBias || (!kEpi && kJ == 4), "deferred stores with a bias: plain 256-column tiles");
   constexpr int kBN = 64 * kJ;  // columns of a tile
   const int n_tiles = tiles_m * tiles_n;
   const int n_items = n_whole + (n_tiles - n_whole) * tail_splits;
@@ -311,12 +314,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
     uint32_t out_off = 0;
     uint32_t rd_off[kJ], gl_off[kJ];  // 192-column tiles: the lane's piece of each read-back and store of a half
     u32x4 rb[kJ];
+    float bv[kJ][4];  // kDeferBias: the bias of the lane's four columns of each column tile
     auto drain_part = [&](int r, int j) __attribute__((always_inline)) {
       uint32_t pk[2];
       float v[4];
       acc_read(acc[r][j], v);
 #pragma unroll
-      for (int c = 0; c < 2; ++c) pk[c] = T::pack2(v[2 * c], v[2 * c + 1]);
+      for (int c = 0; c < 2; ++c) {
+        pk[c] = T::pack2(v[2 * c], v[2 * c + 1]);
+        if constexpr (kDeferBias)  // second rounding, as a separate add on the 16-bit result would do
+          pk[c] = T::pack2(lo_f32<T>(pk[c]) + bv[j][2 * c], hi_f32<T>(pk[c]) + bv[j][2 * c + 1]);
+      }
       *reinterpret_cast<uint2*>(st_w + ((r >> 1) & 1) * kHalfBytes + 16 * (r & 1) * kStageStride + 32 * j) =
           make_uint2(pk[0], pk[1]);
     };
@@ -348,6 +356,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           const uint32_t idx = 64u * k + (uint32_t)lane_e, row = idx / (2 * kJ), piece = idx - row * (2 * kJ);
           rd_off[k] = row * kStageStride + 16u * piece;
           gl_off[k] = (row * (uint32_t)N + (uint32_t)wn + 8u * piece) * 2u;
+        }
+      }
+      if constexpr (kDeferBias) {  // written by the tile that left its sums behind (below)
+        const float* bias_f =
+            reinterpret_cast<const float*>(lds + kXBuffers * kTileBytes + 4 * kStageBytes + wave * kBiasBytes);
+#pragma unroll
+        for (int j = 0; j < kJ; ++j) {
+          const float4 b4 = *reinterpret_cast<const float4*>(bias_f + 16 * j + 4 * (lane_e >> 4));
+          bv[j][0] = b4.x, bv[j][1] = b4.y, bv[j][2] = b4.z, bv[j][3] = b4.w;
         }
       }
 #pragma unroll
@@ -712,9 +729,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
       }
       primed = has_next;
       if constexpr (!kPlanes && !kEpi) {
-        // A tile with all of its rows and columns inside y and no output bias, followed by another whole
-        // tile, leaves its sums in the accumulators: the next tile's first step stores them.
-        if (seq + (int)gridDim.x < end && m0 + BM <= M && n0 + kBN <= N && !out_bias) {
+        // A tile with all of its rows and columns inside y, followed by another whole tile, leaves its sums in
+        // the accumulators: the next tile's first step stores them (a bias: in the kDeferBias instantiation).
+        if (seq + (int)gridDim.x < end && m0 + BM <= M && n0 + kBN <= N && (kDeferBias || !out_bias)) {
+          if constexpr (kDeferBias)
+            *reinterpret_cast<float*>(lds + kXBuffers * kTileBytes + 4 * kStageBytes + wave * kBiasBytes + lane * 4) =
+                T::to_f32(out_bias[n0 + wn + lane]);
           drain_out = out_base;
           pending = true;
           continue;
@@ -766,10 +786,10 @@ int launch_dequant(const uint32_t* wq, const void* scales, const void* biases, i
   return launch_dequant_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
 }
 
-template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4>
+template <typename T, bool kEpi, bool kCut, bool kLowRank, int kJ = 4, bool kDeferBias = false>
 int launch_gemm(const void* x, int64_t M, int64_t K, const void* wfrag, const void* bias, int64_t N, void* y,
                 int n_whole, int splits, float* planes, hipStream_t stream, LowRank lr, Epilogue epi) {
-  auto kernel = frag_gemm_kernel<T, kEpi, kCut, kLowRank, kJ>;
+  auto kernel = frag_gemm_kernel<T, kEpi, kCut, kLowRank, kJ, kDeferBias>;
   static PerDeviceInt configured;
   if (!raise_lds_limit(configured, reinterpret_cast<const void*>(kernel), kLdsBytes)) return MFQ_ELAUNCH;
   const int tiles_m = (int)((M + BM - 1) / BM);
@@ -805,6 +825,12 @@ int launch_gemm_typed(const void* x, int64_t M, int64_t K, const void* copy, con
   }
   if (lr.R) return splits > 1 ? go(no, yes, yes) : go(no, no, yes);  // (no entry point combines update and epilogue)
   if (epi.kind != kEpiNone) return splits > 1 ? go(yes, yes, no) : go(yes, no, no);
+  // with a bias and more than one whole tile to a workgroup: the instantiation whose deferred stores add it (the
+  // one with the K cut's second loop for uncut calls too: without that loop behind it the compiler spills 292
+  // registers on this variant)
+  if (bias && n_whole > compute_units())
+    return launch_gemm<T, false, true, false, 4, true>(x, M, K, copy, bias, N, y, n_whole, splits, planes, stream, lr,
+                                                       epi);
   return splits > 1 ? go(no, yes, no) : go(no, no, no);
 }
 

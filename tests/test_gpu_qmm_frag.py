@@ -171,6 +171,14 @@ def test_two_kernel_path_deferred_stores(oracle, bits, dtype, M, K, N):
     row_inf = np.abs(ref).max(axis=-1, keepdims=True)
     err = np.abs(ys[0].double().cpu().numpy() - ref) / row_inf
     assert err.max() <= TOL, err.max()
+    # A real bias: deferred stores add it (an instantiation of its own).  The same two roundings as a
+    # separate add on the 16-bit result, so y(bias) == round(y(no bias) + bias) bit for bit.
+    bias = to_dev(o._from_f32(seeded(141 + bits, 2, (N,), 0.02), dt), dt)
+    y = torch.full((M, N), float("nan"), dtype=xd.dtype, device="cuda")
+    assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, 64, bits, xd, wd, sd, bd, bias, y, ws, copy) == 0
+    torch.cuda.synchronize()
+    want = (ys[0].float() + bias.float()).to(xd.dtype)
+    assert torch.equal(y.view(torch.int16), want.view(torch.int16))
 
 
 def test_two_kernel_path_epilogues_and_graph_replay(oracle):
