@@ -9,9 +9,13 @@
 //      wavefronts (one per SIMD, 256 rows x 64 columns each), v_mfma_f32_16x16x32
 //      with the weights as the A operand straight from global memory into registers
 //      and x from global memory straight into LDS (three tiles, no registers in
-//      between), persistent workgroups that prefetch across tile boundaries; the
-//      tail of the tile sequence cut along K into float32 planes as in qmm.hip, a
-//      LoRA update as extra k behind the loop, the epilogues of epilogue.h in the store.
+//      between), persistent workgroups that prefetch across tile boundaries and
+//      store a tile's sums behind the first matrix instructions of their next tile;
+//      the tail of the tile sequence cut along K into float32 planes as in qmm.hip, a
+//      LoRA update as extra k behind the loop, the epilogues of epilogue.h in the
+//      store; 192-column tiles where those fit one round of workgroups.
+// Both kernels are also entry points of their own (launch_qmm_frag_copy,
+// launch_qmm_frag_gemm) for weights whose copy the caller keeps.
 // The fused kernel (qmm.hip) dequantises a weight once per 256 rows of x, M / 256
 // times per call, in the shadow of its matrix instructions; here that vector work is
 // gone from the matrix loop, which is what lets it use the 16-cycle instruction shape
