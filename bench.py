@@ -231,6 +231,45 @@ def cpu_baseline(torch, x, wq, s, b, sample_rows):
     }
 
 
+# (configuration, M, K, N, bits) of every GEMM of BASELINE.json's configurations (the matvecs are the bench's own leg)
+CONFIG_SHAPES = (
+    ("1 FLUX to_q", 4096, 3072, 3072, 4),
+    ("3 FLUX single block linear1", 4608, 3072, 21504, 4), ("3 FLUX single block linear2", 4608, 15360, 3072, 4),
+    ("4 Z-Image", 4352, 3840, 3840, 8), ("4 Z-Image", 4352, 3840, 10240, 8), ("4 Z-Image", 4352, 10240, 3840, 8),
+    ("5 Qwen-Image image stream", 6889, 3072, 3072, 4), ("5 Qwen-Image image stream", 6889, 3072, 12288, 4),
+    ("5 Qwen-Image image stream", 6889, 12288, 3072, 4),
+    ("5 Qwen-Image text stream", 256, 3072, 3072, 4), ("5 Qwen-Image text stream", 256, 3072, 12288, 4),
+    ("5 Qwen-Image text stream", 256, 12288, 3072, 4),
+    ("text stream at M = 512", 512, 3072, 3072, 4), ("text stream at M = 512", 512, 3072, 12288, 4),
+    ("text stream at M = 512", 512, 12288, 3072, 4),
+)
+
+
+def config_table(torch, mflux_amd, dev):
+    """Per shape: 100 calls of quantized_matmul back to back, then 100 of torch.matmul
+    on the dequantised weights, each timed as a whole with HIP events (sustained,
+    unlike a short burst; under `rocprofv3 --kernel-trace --stats` the same run
+    gives every kernel's own average)."""
+    rows = []
+    for name, M, K, N, bits in CONFIG_SHAPES:
+        x = seeded_bf16(torch, dev, 3, 0, (M, K), 1.0)
+        w = seeded_bf16(torch, dev, 3, 1, (N, K), 0.02)
+        wq, s, b = mflux_amd.quantize(w, GS, bits)
+        w16 = mflux_amd.dequantize(wq, s, b, GS, bits)
+        del w
+        row = {"config": name, "M": M, "K": K, "N": N, "bits": bits}
+        for key, fn in (("mfq", lambda: mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=bits)),
+                        ("library_bf16", lambda: torch.matmul(x, w16.t()))):
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
+            ms = event_ms(fn, 100, torch)
+            row[key] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M * K * N / ms / 1e9, 1)}
+        rows.append(row)
+        del x, wq, s, b, w16
+    return {"workload": "GEMM shapes of the BASELINE configurations, 100 calls each back to back", "rows": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -246,6 +285,10 @@ def main():
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device-to-device copy, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
+    ap.add_argument("--config-table", action="store_true",
+                    help="instead of the benchmark: every GEMM shape of the BASELINE configurations, each 100 calls "
+                         "back to back (for a kernel trace), with the BLAS library's bf16 GEMM on the dequantised "
+                         "weights beside it; prints one JSON object")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (--gpus 1); nothing is sharded across devices")
@@ -259,6 +302,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(3000)  # for the side legs only; the step's operands are seeded by numpy
+
+    if args.config_table:
+        print(json.dumps(config_table(torch, mflux_amd, dev)))
+        return
 
     if args.calibration_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(7)
