@@ -31,6 +31,7 @@ LINEARS = [
     ("cfg1_flux_to_q", 1, 0, 4096, 3072, 3072, 4, True),
     ("cfg3_flux_single_linear1", 3, 0, 4608, 3072, 21504, 4, True),
     ("cfg3_flux_single_linear2", 3, 1, 4608, 15360, 3072, 4, True),
+    ("cfg3_flux_single_linear1_as_benchmarked_without_bias", 3, 0, 4608, 3072, 21504, 4, False),
     ("cfg4_zimage_attn_3840x3840", 4, 0, 4352, 3840, 3840, 8, False),
     ("cfg4_zimage_ffn_gate_up_3840x10240", 4, 1, 4352, 3840, 10240, 8, False),
     ("cfg4_zimage_ffn_down_10240x3840", 4, 2, 4352, 10240, 3840, 8, False),
