@@ -975,13 +975,27 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const float* __restric
     return;
   }
   const int64_t o = (int64_t)row * N + col;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    if (col + e >= N) break;
+  auto finish = [&](int e) {
     float out = linear(v[e], col + e);
     if (epi.kind == kEpiGelu && col + e >= epi.act_from) out = epi_gelu<T>(out);
     if (epi.kind == kEpiGateResidual)
       out = epi_gate_residual<T>(out, T::to_f32(epi.gate[col + e]), T::to_f32(epi.residual[o + e]));
+    return out;
+  };
+  if ((N & 3) == 0) {  // the quad lies inside the row and is aligned: one store
+    const float out[4] = {finish(0), finish(1), finish(2), finish(3)};
+    if (y_is_f32) {
+      *reinterpret_cast<float4*>(reinterpret_cast<float*>(y) + o) = make_float4(out[0], out[1], out[2], out[3]);
+    } else {
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(y) + o) =
+          make_uint2(T::pack2(out[0], out[1]), T::pack2(out[2], out[3]));
+    }
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (col + e >= N) break;
+    const float out = finish(e);
     if (y_is_f32) {
       reinterpret_cast<float*>(y)[o + e] = out;
     } else {
