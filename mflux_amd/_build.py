@@ -47,20 +47,47 @@ def _compile(src: str) -> str:
 ASM_MFMA_KERNELS = {"qmm_frag.hip": "frag_gemm_kernel"}
 
 
-def check_generated_code(src: str) -> int:
-    """Compiles `src` to assembly (device side) and checks every kernel named in
-    ASM_MFMA_KERNELS for what neither the hardware nor the compiler's hazard
+def _parse_blocks(body: str):
+    """A kernel's listing as basic blocks: [(label, [instruction lines])], split at every label line."""
+    import re
+
+    blocks = [("", [])]
+    for ln in body.split("\n"):
+        s = ln.strip()
+        m = re.match(r"^(\.L[A-Za-z0-9_$.]+):", s)
+        if m:
+            blocks.append((m.group(1), []))
+            continue
+        if not s or s.startswith((";", ".")):
+            continue
+        blocks[-1][1].append(s)
+    return blocks
+
+
+def _wait_states(ins: str) -> int:
+    """What an instruction puts between its neighbours: one issue slot, or the count of an s_nop."""
+    if ins.startswith("s_nop"):
+        return int(ins.split()[1], 0) + 1
+    return 1
+
+
+def check_listing(text: str, kernel_substring: str, where: str = "listing") -> int:
+    """Checks every kernel of the assembly listing `text` whose name contains
+    `kernel_substring` for what neither the hardware nor the compiler's hazard
     recognizer (which does not see matrix instructions written as assembly)
-    would catch, along the listing and across block boundaries:
+    would catch.  (1) and (2) follow the control flow: from each instruction
+    they walk every path through the kernel's basic blocks (fall-through and
+    both ways of each branch, back edges included) until the distance is used
+    up, counting an s_nop by its wait states.
     (1) a read of an accumulation register (v_accvgpr_read, the source of a
     v_accvgpr_mov) or a write of one from outside the matrix pipeline
-    (v_accvgpr_write, the destination of a _mov) must lie at least 24
-    instructions behind the last matrix instruction that wrote that register:
-    the kernels touch accumulators either behind wait states of their own, or
-    (the first pass of a tile, which stores the previous one) some sixty matrix
+    (v_accvgpr_write, the destination of a _mov) must lie at least 24 wait
+    states behind the last matrix instruction that wrote that register: the
+    kernels touch accumulators either behind wait states of their own, or (the
+    first pass of a tile, which stores the previous one) some sixty matrix
     instructions after the register's last update;
-    (2) a matrix instruction that adds to a register must lie at least 4
-    instructions behind a write of that register from outside the pipeline;
+    (2) a matrix instruction that adds to a register must lie at least 4 wait
+    states behind a write of that register from outside the pipeline;
     (3) the body of the k loop may not wait for its loads with a count below 8
     (6 with three column tiles per wavefront instead of four): the weight
     fragments are requested a step and a half ahead with at least nine (six)
@@ -72,8 +99,93 @@ def check_generated_code(src: str) -> int:
     spill a dozen or two outside the k loop; the compiler's choices around the
     assembly have tipped over into hundreds, with accumulators moved between
     the register files, on small changes to the source).
-    Returns the number of kernels checked; raises on a finding."""
+    Returns the number of kernels checked; raises RuntimeError on a finding."""
     import re
+
+    checked = 0
+    for m in re.finditer(r"^(\S*%s\S*):" % re.escape(kernel_substring), text, re.M):
+        name = m.group(1)
+        body = text[m.end():text.index(".Lfunc_end", m.end())]
+        blocks = _parse_blocks(body)
+        index = {label: i for i, (label, _) in enumerate(blocks) if label}
+        col_tiles = re.search(r"ELi(\d)ELb[01]EEEv", name)  # the template argument before the last: column tiles per wavefront
+        least = 2 * int(col_tiles.group(1)) if col_tiles else 8
+
+        def successors(b):
+            ins = blocks[b][1]
+            out = []
+            for s in ins:
+                t = re.match(r"s_c?branch\S*\s+(\S+)", s)
+                if t and t.group(1) in index:
+                    out.append(index[t.group(1)])
+            last = ins[-1] if ins else ""
+            if not (last.startswith("s_branch") or last.startswith("s_endpgm") or last.startswith("s_setpc")):
+                if b + 1 < len(blocks):
+                    out.append(b + 1)
+            return out
+
+        def walk(b, i, budget, visit, seen):
+            """Calls visit(instruction) for everything within `budget` wait states behind instruction i of block b."""
+            ins = blocks[b][1]
+            while budget > 0:
+                i += 1
+                if i >= len(ins):
+                    for nb in successors(b):
+                        if seen.get(nb, 0) < budget:  # not yet entered with as much distance left
+                            seen[nb] = budget
+                            walk(nb, -1, budget, visit, seen)
+                    return
+                visit(ins[i])
+                budget -= _wait_states(ins[i])
+
+        n_matrix = 0
+        for b, (label, ins) in enumerate(blocks):
+            matrix = sum(s.startswith("v_mfma") for s in ins)
+            n_matrix += matrix
+            if matrix >= 128:  # the k loop's body (an item's first step and the low-rank update are blocks of fewer)
+                last_m = max(i for i, s in enumerate(ins) if s.startswith("v_mfma"))
+                short = [int(c) for s in ins[:last_m] for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", s) if int(c) < least]
+                if short:
+                    raise RuntimeError(f"{where}: {name} waits with vmcnt({min(short)}) inside its k loop")
+            for i, s in enumerate(ins):
+                op = s.split()[0]
+                if op.startswith("v_mfma"):
+                    lo, hi = [(int(a), int(c)) for a, c in re.findall(r"a\[(\d+):(\d+)\]", s)][0]
+
+                    def touches(t, lo=lo, hi=hi):
+                        if t.startswith("v_accvgpr"):
+                            for reg in re.findall(r"\ba(\d+)\b", t):
+                                if lo <= int(reg) <= hi:
+                                    raise RuntimeError(f"{where}: {name} touches a{reg} within 24 wait states of a matrix "
+                                                       f"instruction that writes it")
+
+                    walk(b, i, 24, touches, {})
+                elif op.startswith("v_accvgpr_write") or op.startswith("v_accvgpr_mov"):
+                    reg = int(re.findall(r"\ba(\d+)\b", s)[0])
+
+                    def adds(t, reg=reg):
+                        if t.startswith("v_mfma"):
+                            ranges = [(int(a), int(c)) for a, c in re.findall(r"a\[(\d+):(\d+)\]", t)]
+                            if len(ranges) > 1 and ranges[-1][0] <= reg <= ranges[-1][1]:
+                                raise RuntimeError(f"{where}: {name}: a matrix instruction adds to a[{ranges[-1][0]}:"
+                                                   f"{ranges[-1][1]}] within 4 wait states of a write to it")
+
+                    walk(b, i, 4, adds, {})
+        if not n_matrix:
+            raise RuntimeError(f"{where}: {name} holds no matrix instruction; the check does not see the kernel")
+        spills = re.search(r"\.name:\s+%s\n(?:.*\n)*?\s*\.vgpr_spill_count:\s*(\d+)" % re.escape(name), text)
+        if spills is None or int(spills.group(1)) > 48:
+            raise RuntimeError(f"{where}: {name} spills {spills and spills.group(1)} registers (at most 48 expected)")
+        checked += 1
+    if not checked:
+        raise RuntimeError(f"{where}: no kernel named *{kernel_substring}* found")
+    return checked
+
+
+def check_generated_code(src: str) -> int:
+    """Compiles `src` to assembly (device side) and runs check_listing over the
+    kernels named in ASM_MFMA_KERNELS.  Returns the number of kernels checked;
+    raises on a finding."""
     import tempfile
 
     with tempfile.TemporaryDirectory() as tmp:
@@ -83,58 +195,7 @@ def check_generated_code(src: str) -> int:
         if res.returncode != 0:
             raise RuntimeError(f"hipcc -S failed on {src}:\n{res.stdout}\n{res.stderr}")
         text = open(asm).read()
-    checked = 0
-    for m in re.finditer(r"^(\S*%s\S*):" % re.escape(ASM_MFMA_KERNELS[src]), text, re.M):
-        body = text[m.end():text.index(".Lfunc_end", m.end())]
-        n_matrix = 0
-        col_tiles = re.search(r"ELi(\d)ELb[01]EEEv", m.group(1))  # the template argument before the last: column tiles per wavefront
-        least = 2 * int(col_tiles.group(1)) if col_tiles else 8
-        for block in re.split(r"\n\.LBB[0-9_]+:", body):
-            ops = [ln.split()[0] for ln in block.split("\n") if ln.strip() and not ln.strip().startswith((";", "."))]
-            matrix = sum(op.startswith("v_mfma") for op in ops)
-            n_matrix += matrix
-            if matrix >= 128:  # the k loop's body (an item's first step and the low-rank update are blocks of fewer)
-                upto = block[:block.rindex("v_mfma")]  # behind the last one the block may run on into an epilogue
-                short = [int(c) for c in re.findall(r"s_waitcnt vmcnt\((\d+)\)", upto) if int(c) < least]
-                if short:
-                    raise RuntimeError(f"{src}: {m.group(1)} waits with vmcnt({min(short)}) inside its k loop")
-        by_matrix = []  # per instruction: the register range a matrix instruction wrote, else None
-        by_move = []    # per instruction: the register a write from outside the pipeline went to, else None
-        for ln in body.split("\n"):
-            ln = ln.strip()
-            if not ln or ln.startswith((";", ".")):
-                continue
-            op = ln.split()[0]
-            wrote, moved = None, None
-            if op.startswith("v_mfma"):
-                ranges = [(int(a), int(b)) for a, b in re.findall(r"a\[(\d+):(\d+)\]", ln)]
-                wrote = ranges[0]
-                if len(ranges) > 1:  # the addend
-                    lo, hi = ranges[-1]
-                    if any(r is not None and lo <= r <= hi for r in by_move[-4:]):
-                        raise RuntimeError(f"{src}: {m.group(1)}: a matrix instruction adds to a[{lo}:{hi}] within 4 "
-                                           f"instructions of a write to it")
-            elif op.startswith("v_accvgpr"):
-                regs = [int(r) for r in re.findall(r"\ba(\d+)\b", ln)]
-                if op.startswith("v_accvgpr_write"):
-                    moved = regs[0]
-                elif op.startswith("v_accvgpr_mov"):
-                    moved = regs[0]
-                for reg in regs:
-                    if any(r is not None and r[0] <= reg <= r[1] for r in by_matrix[-24:]):
-                        raise RuntimeError(f"{src}: {m.group(1)} touches a{reg} within 24 instructions of a matrix "
-                                           f"instruction that writes it")
-            by_matrix.append(wrote)
-            by_move.append(moved)
-        if not n_matrix:
-            raise RuntimeError(f"{src}: {m.group(1)} holds no matrix instruction; the check does not see the kernel")
-        spills = re.search(r"\.name:\s+%s\n(?:.*\n)*?\s*\.vgpr_spill_count:\s*(\d+)" % re.escape(m.group(1)), text)
-        if spills is None or int(spills.group(1)) > 48:
-            raise RuntimeError(f"{src}: {m.group(1)} spills {spills and spills.group(1)} registers (at most 48 expected)")
-        checked += 1
-    if not checked:
-        raise RuntimeError(f"{src}: no kernel named *{ASM_MFMA_KERNELS[src]}* found")
-    return checked
+    return check_listing(text, ASM_MFMA_KERNELS[src], src)
 
 
 def build_library(verbose: bool = False) -> str:

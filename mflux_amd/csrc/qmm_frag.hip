@@ -371,6 +371,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1, 1))
           bv[j][0] = b4.x, bv[j][1] = b4.y, bv[j][2] = b4.z, bv[j][3] = b4.w;
         }
       }
+      // The first reads of the old tile's sums: this block is entered over the loop's back edge, where no count of
+      // instructions along the listing says how far behind the last matrix instructions are, so the distance is
+      // stated here (32 wait states, more than any matrix instruction needs to retire), on the two row blocks
+      // that are read before the first-pass matrix instructions of this step have put sixty of them in between.
+      if constexpr (kJ == 4) {
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]),
+                       "+a"(acc[1][1]), "+a"(acc[1][2]), "+a"(acc[1][3]));
+      } else {
+        asm volatile("s_nop 15\n\ts_nop 15"
+                     : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[1][0]), "+a"(acc[1][1]),
+                       "+a"(acc[1][2]));
+      }
 #pragma unroll
       for (int j = 0; j < kJ; ++j) drain_part(0, j);
       __builtin_amdgcn_sched_barrier(0);

@@ -226,3 +226,66 @@ def test_generated_code_of_the_assembly_matrix_kernels():
     from mflux_amd import _build
 
     assert _build.check_generated_code("qmm_frag.hip") == 18
+
+
+def _listing(blocks, spills=0):
+    """A synthetic assembly listing of one kernel, `demo_gemm_kernel`, in the
+    form the compiler prints: label lines, one instruction per line, the
+    .Lfunc_end marker and the metadata entry with the spill count."""
+    name = "_Z16demo_gemm_kernelv"
+    lines = [f"{name}:"]
+    for label, ins in blocks:
+        if label:
+            lines.append(f"{label}:")
+        lines += [f"\t{i}" for i in ins]
+    lines += [".Lfunc_end0:", "  - .name:           " + name, f"    .vgpr_spill_count: {spills}", ""]
+    return "\n".join(lines)
+
+
+def test_listing_check_follows_branches():
+    """The distance between a matrix instruction and a read of its accumulator is
+    measured along the control flow, back edges included, with an s_nop counted
+    by its wait states: a loop whose head reads a register that the loop's last
+    matrix instruction wrote is refused although the two lie hundreds of lines
+    apart in the listing, and accepted once the wait states are stated."""
+    from mflux_amd import _build
+
+    mfma = "v_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[4:7], a[0:3]"
+    other = "v_mfma_f32_16x16x32_bf16 a[4:7], v[0:3], v[4:7], a[4:7]"
+    filler = ["v_add_u32_e32 v9, v9, v9"] * 40
+    head_bad = ["v_accvgpr_read_b32 v8, a1"] + filler
+    tail = [other] * 3 + [mfma, "s_cmp_lg_u32 s0, 0", "s_cbranch_scc1 .LBB0_1"]
+    end = [".LBB0_3", ["s_endpgm"]]
+    # straight down the listing the read is 40-odd instructions behind every matrix instruction; over the
+    # back edge it is 3 behind the one that writes a[0:3]
+    bad = _listing([("", filler), (".LBB0_1", head_bad), (".LBB0_2", filler + tail), end])
+    with pytest.raises(RuntimeError, match="touches a1 within 24 wait states"):
+        _build.check_listing(bad, "demo_gemm_kernel")
+    good = _listing([("", filler), (".LBB0_1", ["s_nop 15", "s_nop 15"] + head_bad), (".LBB0_2", filler + tail), end])
+    assert _build.check_listing(good, "demo_gemm_kernel") == 1
+    # a short block between the two does not hide the hazard either
+    hop = _listing([("", filler), (".LBB0_1", head_bad), (".LBB0_2", filler + tail[:-1] + ["s_cbranch_scc1 .LBB0_4"]),
+                    end, (".LBB0_4", ["s_mov_b32 s1, 0", "s_branch .LBB0_1"])])
+    with pytest.raises(RuntimeError, match="touches a1"):
+        _build.check_listing(hop, "demo_gemm_kernel")
+
+
+def test_listing_check_refusals():
+    """The other refusals on synthetic listings: an addend written from outside
+    the matrix pipeline right in front of the instruction, a k loop that waits
+    for its newest loads, too many spills, a listing without the kernel."""
+    from mflux_amd import _build
+
+    mfma = "v_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[4:7], a[0:3]"
+    end = (".LBB0_9", ["s_endpgm"])
+    with pytest.raises(RuntimeError, match="adds to a\\[0:3\\] within 4"):
+        _build.check_listing(_listing([("", ["v_accvgpr_write_b32 a2, v1", "s_nop 1", mfma]), end]), "demo_gemm_kernel")
+    assert _build.check_listing(_listing([("", ["v_accvgpr_write_b32 a2, v1", "s_nop 3", mfma]), end]),
+                                "demo_gemm_kernel") == 1
+    loop = [mfma] * 64 + ["s_waitcnt vmcnt(2)"] + [mfma] * 64
+    with pytest.raises(RuntimeError, match="vmcnt\\(2\\) inside its k loop"):
+        _build.check_listing(_listing([("", loop), end]), "demo_gemm_kernel")
+    with pytest.raises(RuntimeError, match="spills 49"):
+        _build.check_listing(_listing([("", [mfma]), end], spills=49), "demo_gemm_kernel")
+    with pytest.raises(RuntimeError, match="no kernel named"):
+        _build.check_listing(_listing([("", [mfma]), end]), "other_kernel")
