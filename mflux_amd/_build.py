@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libmfq.so")
-SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "qmm_frag.hip", "lora.hip", "norm.hip")
+SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmv_oct.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "qmm_frag.hip", "lora.hip", "norm.hip")
 
 # -ffp-contract=off, correctly rounded division and preserved denormals make
 # the quantize kernel's float32 arithmetic the same IEEE operations as the

@@ -331,6 +331,13 @@ bool qmv_quad_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const vo
 int launch_qmv_quad(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                     hipStream_t stream, bool silu = false);
+// one to four activation rows, 8-bit codes: eight weight rows at a time on the int8 16x16x64 matrix
+// instruction, K split over the eight wavefronts of a workgroup (qmv_oct_covers() says whether it takes a shape)
+bool qmv_oct_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* x, const void* scales,
+                    const void* biases);
+int launch_qmv_oct(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                   const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                   hipStream_t stream, bool silu = false);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
 // low_rank: accumulated with the product by both GEMM kernels (a second kernel

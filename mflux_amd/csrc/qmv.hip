@@ -584,6 +584,10 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                hipStream_t stream) {
   if (M > kRowsPerBlock) return MFQ_EUNSUPPORTED;
+#ifndef MFQ_NO_OCT
+  if (qmv_oct_covers(M, K, N, gs, bits, x, scales, biases))
+    return launch_qmv_oct(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+#endif
   if (qmv_dot_covers(M, K, bits))
     return launch_qmv_dot(x, dtype, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
   // two to four activation rows: four weight rows at a time (for a single row
