@@ -94,7 +94,11 @@ int mfq_dequantize_rows(const uint32_t* wq, const void* scales, const void* bias
 size_t mfq_qmm_t_workspace_bytes(int64_t M, int64_t K, int64_t N, int group_size, int bits) {
   if (check_common(group_size, bits) != MFQ_OK) return 0;
   if (N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
-  if (bits != 4 && bits != 8) return M > 1 ? mfq::qmm_mid_workspace_bytes(M, N, K, group_size) : 0;
+  if (bits != 4 && bits != 8) {
+    if (M <= 1) return 0;
+    if (mfq::prefer_frag_path(M, N, K, group_size, bits)) return mfq::qmm_workspace_bytes(M, N, K, group_size, bits);
+    return mfq::qmm_mid_workspace_bytes(M, N, K, group_size);
+  }
   if (M <= 16) return 0;
   return mfq::qmm_workspace_bytes(M, N, K, group_size, bits);
 }
@@ -191,6 +195,12 @@ int mfq_qmm_t_low_rank(const void* x, int x_dtype, int64_t M, int64_t K, const u
         return rc ? rc : mfq::launch_low_rank_add(x_dtype, low_rank, M, N, y, y_dtype, (hipStream_t)stream);
     }
     if (!mfq::aligned16(y)) return MFQ_EALIGN;
+    // many rows and room for the scratch copy: the two-kernel path of the 4- and 8-bit weights
+    if (M > 16 && K % 64 == 0 && y_dtype == x_dtype && workspace && mfq::aligned16(workspace) &&
+        mfq::qmm_frag_shape_ok(M, N, K, bits) && workspace_bytes >= mfq::qmm_frag_copy_bytes(N, K) &&
+        mfq::prefer_frag_path(M, N, K, group_size, bits))
+      return mfq::launch_qmm(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype, workspace,
+                             workspace_bytes, (hipStream_t)stream, low_rank);
     return mfq::launch_qmm_mid_stream(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                                       workspace, workspace_bytes, (hipStream_t)stream, low_rank);
   }

@@ -363,6 +363,7 @@ size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs);
 // workspace (16-byte aligned): qmm_frag_copy_bytes(N, K) for the copy and, behind it, the float32 planes of a
 // K cut (n_whole whole tiles, the others in `splits` ranges of whole pairs of k steps; splits == 1: no cut)
 bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits);
+bool prefer_frag_path(int64_t M, int64_t N, int64_t K, int gs, int bits);  // where the two-kernel path is the faster
 size_t qmm_frag_copy_bytes(int64_t N, int64_t K);
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,

@@ -1131,11 +1131,19 @@ bool use_mid_kernel(int64_t M, int64_t N, int64_t K) {
   return few_tiles && !(M > 512 && K >= 8192);
 }
 
+#ifndef MFQ_ODD_FRAG_ROWS
+#define MFQ_ODD_FRAG_ROWS 1024
+#endif
+constexpr int64_t kOddBitsFragRows = MFQ_ODD_FRAG_ROWS;
+
 // The two-kernel path (qmm_frag.hip: a 16-bit scratch copy of the weights in fragment order, then a lean
 // GEMM) takes the shapes it wins on: at least eight rows of tiles to spread the copy over.  It cuts K for
 // the tail of the tile sequence by the same plan as the fused kernel.
 bool prefer_frag_path(int64_t M, int64_t N, int64_t K, int gs, int bits) {
-  return M >= 2048 && qmm_frag_shape_ok(M, N, K, bits) && !use_mid_kernel(M, N, K);
+  // (3, 5 and 6 bits: the alternative is the 128-column-tile kernel with its codes cut out of a bit stream,
+  // which the copy overtakes much earlier)
+  const int64_t least_rows = (bits == 4 || bits == 8) ? 2048 : kOddBitsFragRows;
+  return M >= least_rows && qmm_frag_shape_ok(M, N, K, bits) && !use_mid_kernel(M, N, K);
 }
 
 size_t qmm_min_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs) {

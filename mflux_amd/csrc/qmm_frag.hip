@@ -148,6 +148,40 @@ __global__ __launch_bounds__(256) void dequant_frag_kernel(const uint32_t* __res
   }
 }
 
+// The same copy from MLX's 3-, 5- and 6-bit packs, where a row is one little-endian bit stream and 32 codes
+// fill BITS whole words: a wavefront takes two neighbouring blocks per trip (K / 64 is even), lane (u, c16) =
+// (lane / 16, lane % 16) the 32 codes of unit u of the pair's 128 k in row c16 -- BITS words, one scale and one
+// bias (a unit lies in one group) -- and writes their four fragments of 8 values; the 16 lanes of a unit write
+// 256 contiguous bytes per store.
+template <typename T, int GS, int BITS>
+__global__ __launch_bounds__(256) void dequant_frag_stream_kernel(const uint32_t* __restrict__ wq,
+                                                                  const uint16_t* __restrict__ scales,
+                                                                  const uint16_t* __restrict__ biases,
+                                                                  char* __restrict__ out, int N, int K, int n_blocks) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int c16 = lane & 15, u = lane >> 4;
+  const int ks_per_row = K / BK;
+  const int waves = gridDim.x * 4;
+  for (int blk = (blockIdx.x * 4 + threadIdx.x / kWave) * 2; blk < n_blocks; blk += waves * 2) {
+    const int nb = blk / ks_per_row, ks = blk - nb * ks_per_row;
+    const int row = min(nb * 16 + c16, N - 1);  // rows past N repeat the last one; the GEMM never stores their columns
+    const int unit = 2 * ks + u;                // of the row's K / 32
+    const uint32_t* src = wq + (int64_t)row * (K / 32 * BITS) + unit * BITS;
+    uint32_t w[BITS];
+#pragma unroll
+    for (int i = 0; i < BITS; ++i) w[i] = src[i];
+    const int64_t g = (int64_t)row * (K / GS) + (unit * 32) / GS;
+    const float sc = T::to_f32(scales[g]), bi = T::to_f32(biases[g]);
+    char* dst = out + (int64_t)(blk + (u >> 1)) * kBlockBytes + c16 * 16;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {  // codes 8 f .. 8 f + 7 of the unit: k 32 (u % 2) + 8 f of its block
+      const int kk = 32 * (u & 1) + 8 * f;
+      const uint4 v = dequant8_stream<T, BITS>(w, f, sc, bi);
+      *reinterpret_cast<uint4*>(dst + 1024 * ((kk >> 3) & 1) + 256 * (kk >> 4)) = v;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // 2. the GEMM.
 //
@@ -787,7 +821,17 @@ int launch_dequant_bits(const uint32_t* wq, const void* scales, const void* bias
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, wq, (const uint16_t*)scales, (const uint16_t*)biases,
                        (char*)out, (int)N, (int)K, (int)n_blocks);
   };
-  if (bits == 4) {
+  if (bits == 3 || bits == 5 || bits == 6) {
+    const int64_t want = (n_blocks / 2 + 3) / 4;
+    const dim3 stream_grid((unsigned)(want < cap ? want : cap));
+    auto go = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, stream_grid, dim3(256), 0, stream, wq, (const uint16_t*)scales,
+                         (const uint16_t*)biases, (char*)out, (int)N, (int)K, (int)n_blocks);
+    };
+    if (bits == 3) go(dequant_frag_stream_kernel<T, GS, 3>);
+    if (bits == 5) go(dequant_frag_stream_kernel<T, GS, 5>);
+    if (bits == 6) go(dequant_frag_stream_kernel<T, GS, 6>);
+  } else if (bits == 4) {
     if (pair == 4) launch(dequant_frag_kernel<T, GS, 4, 4>); else launch(dequant_frag_kernel<T, GS, 4, 2>);
   } else {
     if (pair == 4) launch(dequant_frag_kernel<T, GS, 8, 4>); else launch(dequant_frag_kernel<T, GS, 8, 2>);
@@ -856,7 +900,8 @@ int launch_gemm_typed(const void* x, int64_t M, int64_t K, const void* copy, con
 bool qmm_frag_shape_ok(int64_t M, int64_t N, int64_t K, int bits) {
   // whole pairs of k steps and at least two of them; whole 16-byte pieces of y; 32-bit byte offsets into x
   // and into the scratch copy
-  return (bits == 4 || bits == 8) && K % (2 * BK) == 0 && K >= 4 * BK && N % 8 == 0 && M * K < ((int64_t)1 << 31) &&
+  return (bits == 3 || bits == 4 || bits == 5 || bits == 6 || bits == 8) && K % (2 * BK) == 0 && K >= 4 * BK &&
+         N % 8 == 0 && M * K < ((int64_t)1 << 31) &&
          ((N + 15) / 16) * 16 * K < ((int64_t)1 << 31);
 }
 

@@ -43,7 +43,10 @@ def _call(lib, name, code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y, ws, ws_b
 @pytest.mark.parametrize("M", [4100, 2400])
 @pytest.mark.parametrize("bits,gs,dtype,with_bias,K", [
     (4, 64, "bf16", True, 512), (8, 64, "bf16", False, 512), (4, 32, "bf16", False, 512), (8, 128, "bf16", True, 512),
-    (4, 128, "f16", True, 512), (8, 32, "f16", False, 512), (4, 64, "bf16", False, 640), (8, 64, "f16", True, 384)])
+    (4, 128, "f16", True, 512), (8, 32, "f16", False, 512), (4, 64, "bf16", False, 640), (8, 64, "f16", True, 384),
+    # 3, 5 and 6 bits: the copy cut out of MLX's bit stream (32 codes to BITS words), then the same GEMM
+    (3, 64, "bf16", True, 512), (5, 32, "bf16", False, 384), (6, 128, "f16", True, 512), (5, 64, "f16", False, 640),
+    (3, 32, "f16", False, 384), (6, 64, "bf16", True, 640)])
 def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_bias, K, M):
     from gpu_util import to_dev, u32_to_dev
     from mflux_amd import _lib
@@ -78,7 +81,7 @@ def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_
     err = np.abs(y.double().cpu().numpy() - ref) / row_inf
     assert err.max() <= TOL, err.max()
 
-    # without a workspace the fused kernel takes the call: same bound, and close to the two-kernel result
+    # without a workspace the fused kernel (for 3, 5 and 6 bits: the 128-column-tile kernel) takes the call: same bound
     y_fused = torch.empty_like(y)
     assert _call(lib, "mfq_qmm_t_ws", code, M, K, N, gs, bits, xd, wd, sd, bd, biasd, y_fused, None, 0) == 0
     torch.cuda.synchronize()
@@ -104,7 +107,10 @@ def test_workspace_tells_the_path():
     cut = q(6889, 3072, 3072, 64, 4) - 3072 * 3072 * 2          # one round + 68 tiles: the tail cut along K
     assert cut > 0 and cut % (68 * plane) == 0
     assert q(1024, 3072, 21504, 64, 4) % plane == 0             # four rows of tiles: the fused kernel (and its cut)
-    assert q(4608, 3072, 21504, 64, 5) == 0                     # odd bit widths have their own kernel
+    assert q(4608, 3072, 21504, 64, 5) == 21504 * 3072 * 2      # 3, 5, 6 bits: the same copy, cut out of the bit stream,
+    rest = q(1024, 3072, 21504, 64, 6) - 21504 * 3072 * 2       # from 1024 rows on (what it replaces there is slower);
+    assert rest > 0 and rest % plane == 0                       # 336 tiles: one round + 80, the tail cut along K
+    assert q(512, 3072, 21504, 64, 3) == 0                      # below: the 128-column-tile kernel, uncut here
 
 
 @pytest.mark.parametrize("bits,dtype", [(4, "bf16"), (8, "f16")])
