@@ -270,6 +270,138 @@ def config_table(torch, mflux_amd, dev):
     return {"workload": "GEMM shapes of the BASELINE configurations, 100 calls each back to back", "rows": rows}
 
 
+def baseline_configs(torch, mflux_amd, dev, quick=False):
+    """BASELINE configurations 1, 4 and 5 as wholes (the headline is configuration 3, the matvec
+    leg configuration 2): the summed time of a configuration's quantized linears, calls back to
+    back on one stream with HIP events around them, and 2MNK of its GEMMs over that time against
+    the dense bf16 peak.  Configuration 5 keeps all 60 blocks' weights resident (11.5 GB of packed
+    4-bit codes, scales and biases, every block its own tensors) and visits them in order, so a
+    block's weights are cold when its linears run; its two modulation matvecs per block are in the
+    time and not in the FLOPs."""
+    from mflux_amd import nn as qnn
+
+    def qlinear(config, index, K, N, bits, bias, w=None):
+        lin = qnn.QuantizedLinear(K, N, bias=bias, group_size=GS, bits=bits)
+        if w is None:
+            w = seeded_bf16(torch, dev, config, index, (N, K), 0.02)
+        lin.weight, lin.scales, lin.biases = mflux_amd.quantize(w, GS, bits)
+        if bias:
+            lin.bias = seeded_bf16(torch, dev, config, index + 500, (N,), 0.02)
+        return lin
+
+    def timed(fn, warm, iters):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        return event_ms(fn, iters, torch)
+
+    out = {}
+    # -- 1: FLUX.1 to_q, 4096 x 3072 -> 3072, W4, bias
+    x = seeded_bf16(torch, dev, 1, 0, (4096, 3072), 1.0)
+    lin = qlinear(1, 1, 3072, 3072, 4, True)
+    ms = timed(lambda: lin(x), 10, 50)
+    flops = 2.0 * 4096 * 3072 * 3072
+    out["config1_flux_to_q_m4096_w4"] = {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
+                                         "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    del lin, x
+
+    # -- 4: Z-Image block, M = 4352, hidden 3840, W8, no bias: q, k, v, out, w1, w3, w2
+    M4 = 4352
+    x = seeded_bf16(torch, dev, 4, 0, (M4, 3840), 1.0)
+    xh = seeded_bf16(torch, dev, 4, 1, (M4, 10240), 1.0)
+    q, k, v, o = (qlinear(4, 10 + i, 3840, 3840, 8, False) for i in range(4))
+    w1, w3 = (qlinear(4, 20 + i, 3840, 10240, 8, False) for i in range(2))
+    w2 = qlinear(4, 30, 10240, 3840, 8, False)
+    flops = 2.0 * M4 * (4 * 3840 * 3840 + 3 * 3840 * 10240)
+
+    def separate():
+        q(x), k(x), v(x), o(x), w1(x), w3(x), w2(xh)
+
+    qkv = qnn.concat_quantized([q, k, v])
+    gate_up = qnn.stack_gate_up(w1, w3)
+
+    def fused():  # q/k/v as one linear; silu(w1 x) * w3 x in the epilogue of one linear over the stacked pair
+        qkv(x), o(x), qnn.swiglu_linear(gate_up, x), w2(xh)
+
+    res = {}
+    for key, fn in (("seven_calls", separate), ("qkv_as_one_and_swiglu_epilogue", fused)):
+        ms = timed(fn, 5, 20)
+        res[key] = {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
+                    "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    out["config4_zimage_block_m4352_w8"] = res
+    del q, k, v, o, w1, w3, w2, qkv, gate_up, x, xh
+
+    # -- 5: Qwen-Image step, 60 blocks, image stream 6889 tokens, text stream 256, W4, bias
+    n_blocks = 6 if quick else 60
+    Mi, Mt = 6889, 256
+    xi, xt = seeded_bf16(torch, dev, 5, 0, (Mi, 3072), 1.0), seeded_bf16(torch, dev, 5, 1, (Mt, 3072), 1.0)
+    xih, xth = seeded_bf16(torch, dev, 5, 2, (Mi, 12288), 1.0), seeded_bf16(torch, dev, 5, 3, (Mt, 12288), 1.0)
+    temb = seeded_bf16(torch, dev, 5, 4, (1, 3072), 1.0)
+    base = {(3072, 3072): seeded_bf16(torch, dev, 5, 10, (3072, 3072), 0.02),
+            (3072, 12288): seeded_bf16(torch, dev, 5, 11, (12288, 3072), 0.02),
+            (12288, 3072): seeded_bf16(torch, dev, 5, 12, (3072, 12288), 0.02),
+            (3072, 18432): seeded_bf16(torch, dev, 5, 13, (18432, 3072), 0.02)}
+    blocks = []
+    for bi in range(n_blocks):
+        def lin(K, N, shift):  # every linear its own weights: the seeded matrix of its shape, rows rotated
+            return qlinear(5, 0, K, N, 4, True, w=torch.roll(base[(K, N)], shifts=7 * (16 * bi + shift) + 1, dims=0))
+        streams = []
+        for st in range(2):
+            attn = [lin(3072, 3072, 8 * st + i) for i in range(4)]
+            streams.append({"q": attn[0], "k": attn[1], "v": attn[2], "out": attn[3],
+                            "qkv": qnn.concat_quantized(attn[:3], share_storage=True),
+                            "mlp_in": lin(3072, 12288, 8 * st + 4), "mlp_out": lin(12288, 3072, 8 * st + 5),
+                            "mod": lin(3072, 18432, 8 * st + 6)})
+        blocks.append(streams)
+    del base
+    resident = sum(t.numel() * t.element_size() for streams in blocks for s_ in streams
+                   for key in ("qkv", "out", "mlp_in", "mlp_out", "mod")
+                   for t in (s_[key].weight, s_[key].scales, s_[key].biases))
+    flops = n_blocks * 2.0 * (Mi + Mt) * (4 * 3072 * 3072 + 2 * 3072 * 12288)
+
+    def step_separate():
+        for streams in blocks:
+            for s_, x_, xh_ in ((streams[0], xi, xih), (streams[1], xt, xth)):
+                qnn.silu_linear(s_["mod"], temb)
+                s_["q"](x_), s_["k"](x_), s_["v"](x_), s_["out"](x_), s_["mlp_in"](x_), s_["mlp_out"](xh_)
+
+    def step_fused():  # q/k/v as one linear
+        for streams in blocks:
+            for s_, x_, xh_ in ((streams[0], xi, xih), (streams[1], xt, xth)):
+                qnn.silu_linear(s_["mod"], temb)
+                s_["qkv"](x_), s_["out"](x_), s_["mlp_in"](x_), s_["mlp_out"](xh_)
+
+    # the same calls with the two streams of tokens on two HIP streams: a block's text-stream linears and
+    # modulation matvecs need nothing from its image-stream linears (the streams meet in the attention, which
+    # is not part of this configuration), and run on the compute units that the image stream's short last
+    # round of tiles leaves idle
+    side = torch.cuda.Stream()
+
+    def step_two_streams():
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            for streams in blocks:
+                s_ = streams[1]
+                qnn.silu_linear(s_["mod"], temb), qnn.silu_linear(streams[0]["mod"], temb)
+                s_["qkv"](xt), s_["out"](xt), s_["mlp_in"](xt), s_["mlp_out"](xth)
+        for streams in blocks:
+            s_ = streams[0]
+            s_["qkv"](xi), s_["out"](xi), s_["mlp_in"](xi), s_["mlp_out"](xih)
+        main.wait_stream(side)
+
+    res = {"blocks": n_blocks, "weights_resident_gb": round(resident / 1e9, 2)}
+    for key, fn in (("sixteen_calls_per_block", step_separate), ("qkv_as_one", step_fused),
+                    ("qkv_as_one_and_text_stream_on_a_second_hip_stream", step_two_streams)):
+        ms = timed(fn, 1, 2 if not quick else 1)
+        res[key] = {"ms_per_step": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
+                    "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    out["config5_qwen_image_step_w4"] = res
+    del blocks
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -282,6 +414,8 @@ def main():
     ap.add_argument("--cpu-sample-rows", type=int, default=2304)
     ap.add_argument("--no-secondary", action="store_true",
                     help="skip the GEMV and quantize measurements (they replay HIP graphs)")
+    ap.add_argument("--configs-quick", action="store_true",
+                    help="the Qwen-Image leg of secondary.configs on 6 blocks instead of 60 (for profiling runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 256 MiB device-to-device copy, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -337,19 +471,36 @@ def main():
         for _, x, wq, s, b in ops:
             mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=BITS)
 
+    # ---- secondary legs on the step's own operands (they run first: the headline below is then timed on a
+    # chip that is already under matrix load, with exactly the requested warm-up steps in front of it) -----
+    #   the library's bf16 GEMM on the same operands
+    library = {}
+    for name, x, wq, s, b in (() if args.no_secondary else ops):
+        w16 = mflux_amd.dequantize(wq, s, b, group_size=GS, bits=BITS)
+        for _ in range(5):  # the library picks and caches its kernel on the first calls
+            torch.matmul(x, w16.t())
+        torch.cuda.synchronize()
+        ms = event_ms(lambda: torch.matmul(x, w16.t()), 20, torch)
+        K, N = x.shape[1], wq.shape[0]
+        library[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
+        del w16
+    #   the same linears on a prepared copy of their weights (the 16-bit copy made once instead of on every
+    #   call, 2 bytes per weight held: the GEMM kernel alone)
+    prepared = {}
+    for name, x, wq, s, b in (() if args.no_secondary else ops):
+        K, N = x.shape[1], wq.shape[0]
+        copy = mflux_amd.prepare_weights(wq, s, b, group_size=GS, bits=BITS)
+        for _ in range(3):
+            mflux_amd.quantized_matmul_prepared(x, copy, N)
+        torch.cuda.synchronize()
+        ms = event_ms(lambda: mflux_amd.quantized_matmul_prepared(x, copy, N), 20, torch)
+        prepared[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1),
+                          "copy_mb_held": round(copy.numel() / 1e6, 1)}
+        del copy
+
+    # ---- the headline: args.warmup untimed steps, then exactly args.steps timed ones ------------------
     for _ in range(args.warmup):
         step()
-    torch.cuda.synchronize()
-    # The chip needs some hundred launches under load before clocks and power settle (the first
-    # batches run up to a tenth slower), so beyond the requested warm-up steps, batches of untimed
-    # steps run until two in a row agree within 1 % (at most 40 batches of 10).
-    settle, prev = [], None
-    for _ in range(40):
-        ms = event_ms(step, 10, torch)
-        settle.append(round(ms, 4))
-        if prev is not None and abs(ms - prev) <= 0.01 * prev:
-            break
-        prev = ms
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     start = torch.cuda.Event(enable_timing=True)
@@ -362,6 +513,16 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms_per_step = start.elapsed_time(stop) / args.steps
+    # Beside it, not in `value`: the same step once batches of ten agree within 1 % (the chip takes
+    # some hundred launches under load before clocks and power settle), and its first batches.
+    settle, prev = [], None
+    for _ in range(40):
+        ms = event_ms(step, 10, torch)
+        settle.append(round(ms, 4))
+        if prev is not None and abs(ms - prev) <= 0.01 * prev:
+            break
+        prev = ms
+    settled_ms = event_ms(step, args.steps, torch)
     # The power sensor is a moving average that needs about half a second to follow the load, far
     # longer than the timed region above: the same step therefore runs on for args.sustain_s
     # seconds right behind it, and power and clock are the samples of the second half of that leg.
@@ -396,7 +557,11 @@ def main():
         "avg_launch_us": round(kernel_ms_per_step * 1e3 / launches, 2),
         "flops_per_launch": flops / launches,
         "sustained": sustained,
-        "settling_ms_per_step": settle,
+        "timed_region": f"{args.warmup} warm-up steps, then {args.steps} timed steps, right behind the "
+                        "library-GEMM and prepared-copy legs on the same operands",
+        "settled": {"ms_per_step": round(settled_ms, 4), "tflops": round(flops / settled_ms / 1e9, 1),
+                    "frac": round(flops / settled_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                    "batches_of_ten_until_two_agree_ms": settle},
     }
 
     # per-shape GEMM timings
@@ -405,32 +570,6 @@ def main():
         ms = event_ms(lambda: mflux_amd.quantized_matmul(x, wq, s, b, group_size=GS, bits=BITS), 20, torch)
         K, N = x.shape[1], wq.shape[0]
         per_shape[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
-
-    # ---- secondary: the library's bf16 GEMM on the same operands ---------------
-    library = {}
-    for name, x, wq, s, b in (() if args.no_secondary else ops):
-        w16 = mflux_amd.dequantize(wq, s, b, group_size=GS, bits=BITS)
-        for _ in range(5):  # the library picks and caches its kernel on the first calls
-            torch.matmul(x, w16.t())
-        torch.cuda.synchronize()
-        ms = event_ms(lambda: torch.matmul(x, w16.t()), 20, torch)
-        K, N = x.shape[1], wq.shape[0]
-        library[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1)}
-        del w16
-
-    # ---- secondary: the same linears on a prepared copy of their weights -------
-    # (the 16-bit copy made once instead of on every call, 2 bytes per weight held: the GEMM kernel alone)
-    prepared = {}
-    for name, x, wq, s, b in (() if args.no_secondary else ops):
-        K, N = x.shape[1], wq.shape[0]
-        copy = mflux_amd.prepare_weights(wq, s, b, group_size=GS, bits=BITS)
-        for _ in range(3):
-            mflux_amd.quantized_matmul_prepared(x, copy, N)
-        torch.cuda.synchronize()
-        ms = event_ms(lambda: mflux_amd.quantized_matmul_prepared(x, copy, N), 20, torch)
-        prepared[name] = {"us": round(ms * 1e3, 1), "tflops": round(2.0 * M_TOKENS * K * N / ms / 1e9, 1),
-                          "copy_mb_held": round(copy.numel() / 1e6, 1)}
-        del copy
 
     # ---- secondary: a rank-16 LoRA on the two linears --------------------------
     # the whole layer (x @ A included) as one fused call against the reference's
@@ -601,6 +740,8 @@ def main():
             2 * 2 * M_TOKENS * 3072 / (fused["layer_norm_modulate_4608x3072"]["fused_us"] * 1e-6) / 1e9 / PEAK_HBM_GBS, 4)
         del xn, scn, shn
 
+    configs = {} if args.no_secondary else baseline_configs(torch, mflux_amd, dev, quick=args.configs_quick)
+
     quant = {}
     for (name, K, N) in (() if args.no_secondary else LINEARS):
         ms = quant_ms[name]
@@ -615,7 +756,7 @@ def main():
     if "w8" in gemv:
         m1 = gemv["w8"]["M1"]
         gemv_traffic, gemv_traffic_source = profiled_traffic("gemv")
-        gemv_roofline = {"kernel": "qmv_dot_kernel<BF16,8,3>", "bound": "hbm", "achieved": m1["GB/s"],
+        gemv_roofline = {"kernel": "qmv_oct_kernel<BF16,3,1>", "bound": "hbm", "achieved": m1["GB/s"],
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": m1["frac_hbm"], "traffic": gemv_traffic,
                          "traffic_source": gemv_traffic_source,
                          "avg_launch_us": m1["us"], "bytes_per_launch": m1["bytes"]}
@@ -640,7 +781,8 @@ def main():
                       "gemv_w8": gemv.get("w8", {}),
                       "gemv_w4": gemv.get("w4", {}), "quantize_w4": quant, "qmm_w4_m512": medium,
                       "qmm_w4_lora_r16": lora, "epilogues_fused_vs_separate": fused,
-                      "library_bf16_gemm_same_operands": library, "qmm_w4_prepared_weights": prepared},
+                      "library_bf16_gemm_same_operands": library, "qmm_w4_prepared_weights": prepared,
+                      "configs": configs},
     }
     if not args.no_cpu_baseline:
         name, x, wq, s, b = ops[0]
