@@ -164,11 +164,16 @@ int mfq_qmm_t(const void* x, int x_dtype, int64_t M, int64_t K,
  *       are the gate projection (w1) and the up projection (w3) in alternating
  *       blocks of 32 rows (N % 64 == 0): nn.silu(self.w1(x)) * self.w3(x) of
  *       src/mflux/models/z_image/model/z_image_transformer/feed_forward.py:13.
- * x, scales, biases, bias and y share one 16-bit type.  Every step rounds to
- * that type where the reference's separate operations would: the linear's
- * output (and its bias add); gelu_approx once (MLX rounds inside it too:
- * parity with MLX unpinned at that level); gate * y, then the sum with the
- * residual; sigmoid, x * sigmoid, then the product with the up projection.
+ * x, scales, biases, bias and y share one 16-bit type.  The linear's output
+ * (and its bias add) is rounded to that type as the reference's linear rounds
+ * it; then gate * y and the sum with the residual, each rounded (the
+ * reference's two operations, bit for bit); sigmoid, x * sigmoid and the
+ * product with the up projection, each rounded (MLX's nn.silu is two
+ * operations).  gelu_approx is evaluated in float32 and rounded ONCE, on
+ * purpose: MLX's nn.gelu_approx is a chain of element-wise operations whose
+ * 16-bit intermediates each round, which is not imitated -- the result is the
+ * correctly rounded value of the formula, a few units in the last place from
+ * the reference's (parity with MLX unpinned at that level).
  * MFQ_EUNSUPPORTED for M <= 16 (the matvec kernels have no epilogue), N % 8 != 0,
  * and, with 256 x 256 tiles, shapes without whole scale periods (K/64 not a
  * multiple of 4 * group_size / 64): run mfq_qmm_t and apply the operations.

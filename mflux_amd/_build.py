@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.path.join(CSRC, "libmfq.so")
-SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmv_oct.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "qmm_frag.hip", "lora.hip", "norm.hip")
+SOURCES = ("abi.hip", "quantize.hip", "qmv.hip", "qmv_dot.hip", "qmv_quad.hip", "qmv_odd.hip", "qmv_oct.hip", "qmv_oct4.hip", "qmm.hip", "qmm_epi.hip", "qmm_mid.hip", "qmm_mid_stream.hip", "qmm_n.hip", "qmm_frag.hip", "lora.hip", "norm.hip")
 
 # -ffp-contract=off, correctly rounded division and preserved denormals make
 # the quantize kernel's float32 arithmetic the same IEEE operations as the
@@ -221,7 +221,7 @@ def sanitize_abi(verbose: bool = False) -> str:
     """Host-sanitizer run of the C ABI's argument validation: abi.hip compiled
     with AddressSanitizer and UndefinedBehaviorSanitizer on its host side (the
     device side is untouched), linked with the ordinary kernel objects and the
-    driver csrc/abi_sanitize_check.cpp, and run.  Every call in the driver is
+    driver tests/abi_sanitize_check.cpp, and run.  Every call in the driver is
     refused before a launch, so no GPU is needed.  Needs the objects of
     build_library().  Returns the driver's output; raises if it reports a
     finding."""
@@ -239,7 +239,7 @@ def sanitize_abi(verbose: bool = False) -> str:
     steps = [
         [hipcc(), *HIPCC_FLAGS, *host_san, "-c", os.path.join(CSRC, "abi.hip"), "-o", abi_o],
         [hipcc(), "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-c",
-         os.path.join(CSRC, "abi_sanitize_check.cpp"), "-o", drv_o],
+         os.path.join(os.path.dirname(os.path.dirname(CSRC)), "tests", "abi_sanitize_check.cpp"), "-o", drv_o],
         [hipcc(), "--offload-arch=gfx950", "-fsanitize=address,undefined", "-o", exe, drv_o, abi_o, *others],
     ]
     for cmd in steps:

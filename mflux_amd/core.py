@@ -240,16 +240,39 @@ def quantized_matmul(x: torch.Tensor, w: torch.Tensor, scales: torch.Tensor, bia
 
 
 
+class PreparedWeights:
+    """What :func:`prepare_weights` returns: the 16-bit copy (``data``, an opaque
+    uint8 tensor) together with what it was made from -- the dtype of the values,
+    the weight's ``output_dims`` x ``input_dims``, ``group_size`` and ``bits`` --
+    so that :func:`quantized_matmul_prepared` can refuse an ``x`` of another dtype
+    or width instead of multiplying it with bytes that mean something else (a
+    bfloat16 and a float16 copy of one shape have the same size)."""
+
+    __slots__ = ("data", "dtype", "output_dims", "input_dims", "group_size", "bits")
+
+    def __init__(self, data, dtype, output_dims, input_dims, group_size, bits):
+        self.data, self.dtype = data, dtype
+        self.output_dims, self.input_dims = int(output_dims), int(input_dims)
+        self.group_size, self.bits = int(group_size), int(bits)
+
+    def numel(self) -> int:
+        return self.data.numel()
+
+    def __repr__(self) -> str:
+        return (f"PreparedWeights({self.output_dims} x {self.input_dims}, {self.dtype}, group_size={self.group_size}, "
+                f"bits={self.bits}, {self.data.numel()} bytes on {self.data.device})")
+
+
 def prepare_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor, group_size: int = 64,
-                    bits: int = 4) -> torch.Tensor | None:
+                    bits: int = 4) -> PreparedWeights | None:
     """The 16-bit copy of ``dequantize(w)`` that a large ``quantized_matmul``
     makes on every call, made once: for weights that do not change between calls
     and a caller with 2 bytes per weight of device memory to spare
     (``include/mfq.h``: ``mfq_qmm_t_prepare``).  Not part of MLX, which
-    dequantises inside every ``mx.quantized_matmul``.  Returns an opaque uint8
-    tensor for ``quantized_matmul_prepared``, or ``None`` where the library has
-    no such copy for the shape (bits other than 4 or 8, ``K`` not a multiple of
-    128, ``N`` not a multiple of 8).  The values are those every other kernel
+    dequantises inside every ``mx.quantized_matmul``.  Returns a
+    :class:`PreparedWeights` for ``quantized_matmul_prepared``, or ``None`` where
+    the library has no such copy for the shape (``K`` not a multiple of 128,
+    ``N`` not a multiple of 8).  The values are those every other kernel
     multiplies with: one rounding of ``fma(code, scale, bias)`` to the dtype of
     ``scales``."""
     _check_group_bits("prepare_weights", group_size, bits)
@@ -269,24 +292,30 @@ def prepare_weights(w: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
                                    group_size, bits, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise _lib.MfqError("mfq_qmm_t_prepare", rc, lib.mfq_strerror(rc).decode())
-    return out
+    return PreparedWeights(out, scales.dtype, N, K, group_size, bits)
 
 
-def quantized_matmul_prepared(x: torch.Tensor, prepared: torch.Tensor, output_dims: int,
+def quantized_matmul_prepared(x: torch.Tensor, prepared: PreparedWeights, output_dims: int | None = None,
                               bias: torch.Tensor | None = None) -> torch.Tensor:
     """``x @ dequantize(w).T (+ bias)`` on the copy ``prepare_weights`` made of
     ``w``: the second kernel of a large ``quantized_matmul`` alone, with the same
     bits in its result.  ``x``: ``[..., K]`` of the 16-bit dtype the copy was
     made in (the dtype of the scales); any number of rows, meant for some
     thousands (below that ``quantized_matmul``'s other kernels are the faster
-    ones).  Inference only."""
-    if x.dtype not in (torch.float16, torch.bfloat16):
-        raise ValueError(f"[quantized_matmul_prepared] x must be float16 or bfloat16, got {x.dtype}")
+    ones).  ``output_dims``, if given, must be the copy's.  Inference only."""
+    if not isinstance(prepared, PreparedWeights):
+        raise ValueError("[quantized_matmul_prepared] `prepared` must be what prepare_weights returned")
+    if x.dtype != prepared.dtype:
+        raise ValueError(f"[quantized_matmul_prepared] the copy holds {prepared.dtype} values, x is {x.dtype}")
     _require_hip("quantized_matmul_prepared", x, "x")
     lib = _lib.load()
-    N, K = int(output_dims), x.shape[-1]
-    if prepared.dtype != torch.uint8 or prepared.numel() != lib.mfq_qmm_t_prepared_bytes(N, K, 4):
-        raise ValueError(f"[quantized_matmul_prepared] the prepared copy does not belong to a weight of {N} x {K}")
+    N, K = prepared.output_dims, x.shape[-1]
+    if K != prepared.input_dims or (output_dims is not None and int(output_dims) != N):
+        raise ValueError(f"[quantized_matmul_prepared] the prepared copy belongs to a weight of {N} x "
+                         f"{prepared.input_dims}, not {output_dims if output_dims is not None else N} x {K}")
+    if prepared.data.device != x.device:
+        raise ValueError("[quantized_matmul_prepared] x and the prepared copy are on different devices")
+    prepared = prepared.data
     lead = tuple(x.shape[:-1])
     x2 = x.reshape(-1, K).contiguous()
     M = x2.shape[0]

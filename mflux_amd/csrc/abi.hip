@@ -280,6 +280,9 @@ int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
   if (mfq::qmv_oct_covers(M, K, N, group_size, bits, x, scales, biases))
     return mfq::launch_qmv_oct(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
                                (hipStream_t)stream, true);
+  if (mfq::qmv_oct4_covers(M, K, N, group_size, bits, x, scales, biases))
+    return mfq::launch_qmv_oct4(x, x_dtype, M, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,
+                                (hipStream_t)stream, true);
 #endif
   if (mfq::qmv_dot_covers(M, K, bits))
     return mfq::launch_qmv_dot(x, x_dtype, K, wq, scales, biases, bias, N, group_size, bits, y, y_dtype,

@@ -338,6 +338,12 @@ bool qmv_oct_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const voi
 int launch_qmv_oct(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                    hipStream_t stream, bool silu = false);
+// the same for 4-bit codes (qmv_oct4.hip)
+bool qmv_oct4_covers(int64_t M, int64_t K, int64_t N, int gs, int bits, const void* x, const void* scales,
+                     const void* biases);
+int launch_qmv_oct4(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
+                    const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
+                    hipStream_t stream, bool silu = false);
 // workspace: optional float32 scratch for the K-split of shapes with few output
 // tiles (qmm_workspace_bytes() says how much; without it K is not split)
 // low_rank: accumulated with the product by both GEMM kernels (a second kernel

@@ -13,12 +13,19 @@
 //                     rows: g(c) = 64 (c / 32) + c % 32, u(c) = g(c) + 32
 //                     (src/mflux/models/z_image/model/z_image_transformer/
 //                     feed_forward.py:13: w2(silu(w1 x) * w3 x)); y is [M, N / 2].
-// Every step rounds to the 16-bit type T where the reference's separate
-// element-wise operations would: the linear's output (and its bias add), then
-//   gelu: one rounding of the float32 evaluation;
-//   gate/residual: the product gate * y, then the sum;
+// The linear's output (and its bias add) is rounded to the 16-bit type T as the
+// reference's linear rounds it; behind that
+//   gate/residual: the product gate * y is rounded, then the sum -- the two
+//           element-wise operations of the reference, bit for bit;
 //   swiglu: sigmoid, x * sigmoid (MLX's nn.silu is those two operations), then
-//           the product with the up projection.
+//           the product with the up projection, each rounded;
+//   gelu:   evaluated in float32 and rounded ONCE.  This is a deliberate
+//           departure: MLX's nn.gelu_approx is a chain of some eight element-wise
+//           operations whose 16-bit intermediates each round, which this does not
+//           imitate (the chain's exact order inside MLX is not on record here, so
+//           imitating it would pin nothing).  The result is the correctly rounded
+//           value of the formula, a few units in the last place from what the
+//           reference's chain gives.
 #pragma once
 
 #include "common.h"

@@ -587,6 +587,8 @@ int launch_qmv(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* w
 #ifndef MFQ_NO_OCT
   if (qmv_oct_covers(M, K, N, gs, bits, x, scales, biases))
     return launch_qmv_oct(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
+  if (qmv_oct4_covers(M, K, N, gs, bits, x, scales, biases))
+    return launch_qmv_oct4(x, dtype, M, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);
 #endif
   if (qmv_dot_covers(M, K, bits))
     return launch_qmv_dot(x, dtype, K, wq, scales, biases, bias, N, gs, bits, y, y_dtype, stream);

@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import contextlib
 import math
+import weakref
 from typing import Callable
 
 import torch
@@ -97,7 +98,19 @@ class QuantizedLinear(torch.nn.Module):
     PREPARED_MIN_ROWS = 2048  # from here on forward() multiplies with the prepared copy, if there is one
 
     def _weights_key(self):
-        return tuple((t.data_ptr(), t._version) for t in (self.weight, self.scales, self.biases))
+        # weak references, not addresses: a fresh tensor can reuse a freed tensor's address at version 0
+        return tuple((weakref.ref(t), t._version) for t in (self.weight, self.scales, self.biases))
+
+    def _prepared_is_current(self) -> bool:
+        key = getattr(self, "_prepared_key", None)
+        now = (self.weight, self.scales, self.biases)
+        return key is not None and all(ref() is t and version == t._version for (ref, version), t in zip(key, now))
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to() / .cuda() / .half(): the kept copy belongs to the old tensors
+        self._prepared = None
+        self._prepared_key = None
+        return super()._apply(fn, *args, **kwargs)
 
     def prepare(self) -> bool:
         """Keeps a 16-bit copy of the dequantised weights in the order the large-M
@@ -114,7 +127,7 @@ class QuantizedLinear(torch.nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if (getattr(self, "_prepared", None) is not None and x.dtype == self.scales.dtype and x.shape[-1] > 0
                 and x.numel() // x.shape[-1] >= self.PREPARED_MIN_ROWS and not (torch.is_grad_enabled() and x.requires_grad)):
-            if self._prepared_key != self._weights_key():
+            if not self._prepared_is_current():
                 self.prepare()
             if self._prepared is not None:
                 return core.quantized_matmul_prepared(x, self._prepared, self.output_dims, self.bias)
@@ -210,7 +223,19 @@ def gate_residual_linear(layer: torch.nn.Module, x: torch.Tensor, gate: torch.Te
     feature (``[N]`` or ``[1, N]``): ``residual + gate * proj_out(.)`` of a
     single-stream block (single_transformer_block.py:45,57) and ``hidden + gate *
     ff(.)`` / ``hidden + gate * attn_output`` of a joint block
-    (joint_transformer_block.py:84-90).  A float layer gets the composed form."""
+    (joint_transformer_block.py:84-90).  The reference's gate is one vector per
+    batch entry, expanded over the sequence (``mx.expand_dims(gate, 1)``): a
+    ``gate`` of shape ``[B, N]`` or ``[B, 1, N]`` next to ``x`` of ``[B, S, K]``
+    runs the kernel once per batch entry, each with its own vector.  A float
+    layer gets the composed form."""
+    N = layer.output_dims if isinstance(layer, QuantizedLinear) else layer.weight.shape[0]
+    if gate.numel() != N:
+        B = x.shape[0] if x.ndim >= 3 else 0
+        if B and gate.numel() == B * N and tuple(gate.shape) in ((B, N), (B, 1, N)) and residual.shape[0] == B:
+            gates = gate.reshape(B, N)
+            return torch.stack([gate_residual_linear(layer, x[i], gates[i], residual[i]) for i in range(B)])
+        raise ValueError(f"[gate_residual_linear] gate must hold {N} values, or {N} per batch entry as [B, {N}] or "
+                         f"[B, 1, {N}] next to x of [B, S, K]; got {tuple(gate.shape)} for x of {tuple(x.shape)}")
     if not isinstance(layer, QuantizedLinear):
         return residual + gate.reshape(-1) * layer(x)
     w, s, b = _linear_parts(layer, "gate_residual_linear")

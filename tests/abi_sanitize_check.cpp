@@ -10,7 +10,7 @@
 #include <cstdlib>
 #include <cstring>
 
-#include "../../include/mfq.h"
+#include "../include/mfq.h"
 
 static int failures = 0;
 static void expect(const char* what, int got, int want) {
@@ -100,7 +100,7 @@ int main() {
   expect("prepare: dtype", mfq_qmm_t_prepare(u, p, p, MFQ_F32, 64, 256, 64, 4, p, nullptr), MFQ_EDTYPE);
   expect("prepare: K", mfq_qmm_t_prepare(u, p, p, MFQ_BF16, 64, 250, 64, 4, p, nullptr), MFQ_ESHAPE);
   expect("prepare: null", mfq_qmm_t_prepare(u, p, nullptr, MFQ_BF16, 64, 256, 64, 4, p, nullptr), MFQ_ENULL);
-  expect("prepare: bits", mfq_qmm_t_prepare(u, p, p, MFQ_BF16, 64, 256, 64, 6, p, nullptr), MFQ_EUNSUPPORTED);
+  expect("prepare: K", mfq_qmm_t_prepare(u, p, p, MFQ_BF16, 64, 192, 64, 4, p, nullptr), MFQ_EUNSUPPORTED);
   expect("prepared: dtype", mfq_qmm_t_prepared(p, MFQ_F32, 4, 256, p, nullptr, 64, p, nullptr, 0, nullptr), MFQ_EDTYPE);
   expect("prepared: M", mfq_qmm_t_prepared(p, MFQ_BF16, 0, 256, p, nullptr, 64, p, nullptr, 0, nullptr), MFQ_ESHAPE);
   expect("prepared: null", mfq_qmm_t_prepared(p, MFQ_BF16, 4, 256, nullptr, nullptr, 64, p, nullptr, 0, nullptr), MFQ_ENULL);

@@ -136,14 +136,15 @@ def test_argument_validation_needs_no_device():
     # the two halves of the large-M call apart: which shapes have a prepared copy, and the checks of both calls
     nbytes = lib.mfq_qmm_t_prepared_bytes
     assert nbytes(3072, 3072, 4) == 3072 * 3072 * 2 and nbytes(3208, 512, 8) == 3216 * 512 * 2
-    assert nbytes(3072, 3072, 5) == 0 and nbytes(3072, 192, 4) == 0 and nbytes(3076, 512, 4) == 0 and nbytes(0, 512, 4) == 0
+    assert nbytes(3072, 3072, 5) == 3072 * 3072 * 2     # 3, 5 and 6 bits have the same copy
+    assert nbytes(3072, 3072, 7) == 0 and nbytes(3072, 192, 4) == 0 and nbytes(3076, 512, 4) == 0 and nbytes(0, 512, 4) == 0
     prep = lib.mfq_qmm_t_prepare
     assert prep(base, base, base, _lib.F32, 64, 256, 64, 4, base, None) == E["dtype"]
     assert prep(base, base, base, _lib.BF16, 64, 256, 48, 4, base, None) == E["group"]
     assert prep(base, base, base, _lib.BF16, 64, 250, 64, 4, base, None) == E["shape"]
     assert prep(base, base, None, _lib.BF16, 64, 256, 64, 4, base, None) == E["null"]
     assert prep(base, base, base, _lib.BF16, 64, 256, 64, 4, base + 8, None) == E["align"]
-    assert prep(base, base, base, _lib.BF16, 64, 256, 64, 6, base, None) == E["unsupported"]
+    assert prep(base, base, base, _lib.BF16, 64, 192, 64, 4, base, None) == E["unsupported"]   # K not whole pairs of steps
     prepared = lib.mfq_qmm_t_prepared
     assert prepared(base, _lib.F32, 4, 256, base, None, 64, base, None, 0, None) == E["dtype"]
     assert prepared(base, _lib.BF16, 0, 256, base, None, 64, base, None, 0, None) == E["shape"]
@@ -207,7 +208,7 @@ def test_torch_ops_are_registered_and_refuse_cpu_tensors():
 def test_abi_validation_clean_under_host_sanitizers():
     """The C ABI's argument validation (csrc/abi.hip, host side) under
     AddressSanitizer and UndefinedBehaviorSanitizer: every refusal of
-    csrc/abi_sanitize_check.cpp comes back with its status and no finding."""
+    tests/abi_sanitize_check.cpp comes back with its status and no finding."""
     from mflux_amd import _build
 
     assert "every refusal clean" in _build.sanitize_abi()

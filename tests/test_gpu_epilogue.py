@@ -166,6 +166,16 @@ def test_epilogue_module_helpers_and_composed_paths(oracle):
         assert torch.equal(qnn.gate_residual_linear(q1, x, gate, res), res + gate * q1(x))
         assert _ulps_apart(qnn.gelu_linear(q1, x), mflux_amd.gelu_approx(q1(x))) <= 1.01
         assert torch.equal(qnn.gate_residual_linear(w1, x, gate, res), res + gate * w1(x))  # float layer: composed
+        # one gate vector per batch entry, expanded over the sequence as the reference does
+        # (joint_transformer_block.py:84-90: mx.expand_dims(gate, 1)): [B, N] and [B, 1, N] next to x of [B, S, K]
+        xb = torch.stack([x, x.flip(0)])
+        resb = torch.stack([res, res.flip(0)])
+        gates = torch.stack([gate.reshape(-1), gate.reshape(-1).flip(0)])
+        want = torch.stack([resb[i] + gates[i] * q1(xb[i]) for i in range(2)])   # (per entry: the same kernel as above)
+        assert torch.equal(qnn.gate_residual_linear(q1, xb, gates, resb), want)
+        assert torch.equal(qnn.gate_residual_linear(q1, xb, gates[:, None, :], resb), want)
+        with pytest.raises(ValueError, match="per batch entry"):
+            qnn.gate_residual_linear(q1, xb, gates[:, :8], resb)
     x32 = torch.randn(40, K, device="cuda")
     y = mflux_amd.quantized_matmul_epilogue(x32, q1.weight, q1.scales, q1.biases, epilogue="gelu", bits=8)
     assert y.dtype == torch.float32

@@ -338,11 +338,29 @@ def test_quantized_linear_prepare():
     y1 = mflux_amd.quantized_matmul(x, w2, sc2, b2, bias=lin.bias)
     assert not torch.equal(y1, y0)
     assert torch.equal(lin(x), y1)
+    # 3, 5 and 6 bits have the same copy (cut out of the bit stream); a width the copy is not built for has none
     odd = mflux_amd.nn.QuantizedLinear(512, 3072, bias=False, group_size=64, bits=6, device="cuda")
-    assert not odd.prepare()
-    assert odd(x).shape == (2, 2304, 3072)
+    y_odd = odd(x)
+    assert odd.prepare() and torch.equal(odd(x), y_odd)
+    narrow = mflux_amd.nn.QuantizedLinear(192, 3072, bias=False, group_size=64, bits=4, device="cuda")
+    assert not narrow.prepare()
+    # the copy knows what it was made from: another dtype or width is refused, not multiplied
+    copy = mflux_amd.prepare_weights(lin.weight, lin.scales, lin.biases, 64, 4)
+    assert (copy.dtype, copy.output_dims, copy.input_dims, copy.bits) == (torch.bfloat16, 3072, 512, 4)
+    with pytest.raises(ValueError, match="holds torch.bfloat16"):
+        mflux_amd.quantized_matmul_prepared(x.half(), copy)
+    with pytest.raises(ValueError, match="belongs to a weight of 3072 x 512"):
+        mflux_amd.quantized_matmul_prepared(x[..., :256].contiguous(), copy)
+    with pytest.raises(ValueError, match="what prepare_weights returned"):
+        mflux_amd.quantized_matmul_prepared(x, copy.data)
+    assert torch.equal(mflux_amd.quantized_matmul_prepared(x, copy, bias=lin.bias), lin(x))
+    # a tensor assigned afresh (not written into) is noticed too, whatever address it gets
+    lin.prepare()
+    lin.weight = w2.clone()
+    assert not lin._prepared_is_current()
+    assert torch.equal(lin(x), y1) and lin._prepared_is_current()
     # the walk over a model: every quantized linear that has such a copy, and what they hold together
     model = torch.nn.Sequential(mflux_amd.nn.QuantizedLinear(512, 1024, device="cuda"), torch.nn.GELU(),
-                                mflux_amd.nn.QuantizedLinear(1024, 512, bits=8, device="cuda"), odd)
-    assert mflux_amd.nn.prepare(model) == 2 * (1024 * 512 + 512 * 1024)
-    assert mflux_amd.nn.prepare(model, min_output_dims=1024) == 2 * 1024 * 512
+                                mflux_amd.nn.QuantizedLinear(1024, 512, bits=8, device="cuda"), odd, narrow)
+    assert mflux_amd.nn.prepare(model) == 2 * (1024 * 512 + 512 * 1024 + 3072 * 512)
+    assert mflux_amd.nn.prepare(model, min_output_dims=1024) == 2 * (1024 * 512 + 3072 * 512)
