@@ -207,6 +207,24 @@ int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* 
               int y_dtype, void* stream);
 
 /*
+ * mfq_qmm_n with an optional workspace; the same reference call
+ * (mx.quantized_matmul(..., transpose=False), the input gradient of the
+ * quantized linears that target_injector.py:30-33 wraps).  With
+ * mfq_qmm_n_workspace_bytes(M, N, K, group_size, bits) bytes of 16-byte aligned
+ * device memory (0: the shape does not use any), calls with many rows of x, 4-
+ * or 8-bit weights and a 16-bit y run as two kernels: a 16-bit copy of the
+ * dequantised weight, transposed into the order the matrix instructions
+ * consume, then the GEMM of mfq_qmm_t's large-M path on it (about twice the
+ * rate of the one-kernel form).  The workspace may be reused by the next call
+ * on the same stream.  With a smaller workspace, or none, the call is
+ * mfq_qmm_n.
+ */
+size_t mfq_qmm_n_workspace_bytes(int64_t M, int64_t N, int64_t K, int group_size, int bits);
+int mfq_qmm_n_ws(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                 const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y, int y_dtype,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * mfq_qmm_t with an optional float32 workspace.  Has no counterpart in the
  * reference (MLX allocates inside its ops).  Shapes whose output tiles do not
  * fill the GPU's compute units -- the text-stream linears of the double

@@ -28,6 +28,9 @@ SIGNATURES = {
     "mfq_qmm_t_epilogue": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _INT, _PTR, _PTR,
                                   _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),
     "mfq_qmm_n": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _I64, _INT, _INT, _PTR, _INT, _PTR]),
+    "mfq_qmm_n_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
+    "mfq_qmm_n_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _I64, _INT, _INT, _PTR, _INT, _PTR,
+                            ctypes.c_size_t, _PTR]),
     "mfq_qmm_t_workspace_bytes": (ctypes.c_size_t, [_I64, _I64, _I64, _INT, _INT]),
     "mfq_qmm_t_ws": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR,
                             ctypes.c_size_t, _PTR]),

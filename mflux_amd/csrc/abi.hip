@@ -255,6 +255,18 @@ int mfq_qmm_t_epilogue(const void* x, int x_dtype, int64_t M, int64_t K, const u
 
 int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
               const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y, int y_dtype, void* stream) {
+  return mfq_qmm_n_ws(x, x_dtype, M, N, wq, scales, biases, sb_dtype, K, group_size, bits, y, y_dtype, nullptr, 0, stream);
+}
+
+size_t mfq_qmm_n_workspace_bytes(int64_t M, int64_t N, int64_t K, int group_size, int bits) {
+  if (check_common(group_size, bits) != MFQ_OK) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || K % group_size || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  return mfq::qmm_n_workspace_bytes(M, N, K, group_size, bits);
+}
+
+int mfq_qmm_n_ws(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                 const void* biases, int sb_dtype, int64_t K, int group_size, int bits, void* y, int y_dtype,
+                 void* workspace, size_t workspace_bytes, void* stream) {
   if (int rc = check_common(group_size, bits)) return rc;
   if (!is16(x_dtype) || x_dtype != sb_dtype) return MFQ_EDTYPE;
   if (y_dtype != sb_dtype && y_dtype != MFQ_F32) return MFQ_EDTYPE;
@@ -262,7 +274,8 @@ int mfq_qmm_n(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_t* 
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX || N * (K * bits / 32) >= (int64_t)1 << 31) return MFQ_ESHAPE;
   if (!x || !wq || !scales || !biases || !y) return MFQ_ENULL;
   if (!mfq::aligned16(x) || !mfq::aligned16(wq) || !mfq::aligned16(y)) return MFQ_EALIGN;
-  return mfq::launch_qmm_n(x, x_dtype, M, N, wq, scales, biases, K, group_size, bits, y, y_dtype, (hipStream_t)stream);
+  return mfq::launch_qmm_n_ws(x, x_dtype, M, N, wq, scales, biases, K, group_size, bits, y, y_dtype, workspace,
+                              workspace_bytes, (hipStream_t)stream);
 }
 
 int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,

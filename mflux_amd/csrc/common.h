@@ -374,6 +374,18 @@ size_t qmm_frag_copy_bytes(int64_t N, int64_t K);
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                     const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, void* workspace,
                     int n_whole, int splits, hipStream_t stream, LowRank low_rank, Epilogue epi);
+// the same path for the weight not transposed, y[M, K] = x[M, N] @ dequantize(wq[N, K]): the copy holds W^T
+// (qmm_frag_copy_bytes(K, N) of workspace, the planes of a K cut wherever `planes` points)
+bool qmm_frag_n_shape_ok(int64_t M, int64_t N, int64_t K, int bits);
+int launch_qmm_frag_n(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                      const void* biases, int64_t K, int gs, int bits, void* y, void* workspace, float* planes,
+                      int n_whole, int splits, hipStream_t stream);
+// y[M, K] = x[M, N] @ dequantize(wq[N, K]) with an optional workspace: with qmm_n_workspace_bytes() of it the
+// two-kernel path takes the shapes it is the faster on, without it (or elsewhere) launch_qmm_n runs
+size_t qmm_n_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits);
+int launch_qmm_n_ws(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                    const void* biases, int64_t K, int gs, int bits, void* y, int y_dtype, void* workspace,
+                    size_t workspace_bytes, hipStream_t stream);
 // its two halves apart: the copy alone (weights that do not change between calls need it once), and the GEMM on a
 // copy made before, with the planes of a K cut wherever the caller has room for them
 int launch_qmm_frag_copy(int dtype, const uint32_t* wq, const void* scales, const void* biases, int64_t N, int64_t K,

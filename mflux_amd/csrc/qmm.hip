@@ -1208,6 +1208,33 @@ int launch_qmm_prepared(const void* x, int dtype, int64_t M, int64_t K, const vo
                               plan.splits, stream, LowRank(), Epilogue());
 }
 
+// The untransposed product on the two-kernel path: from 1024 rows of x on (the kernel it replaces there,
+// qmm_n.hip, runs at half the rate), where the transposed copy exists and the GEMM's tiles fill the chip.
+static bool prefer_frag_n(int64_t M, int64_t N, int64_t K, int bits) {
+  return M >= 1024 && qmm_frag_n_shape_ok(M, N, K, bits) && !use_mid_kernel(M, K, N);
+}
+
+size_t qmm_n_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits) {
+  if (!prefer_frag_n(M, N, K, bits)) return 0;
+  return qmm_frag_copy_bytes(K, N) + tail_plane_bytes(M, K, plan_tail(M, K, N, 2, compute_units()));
+}
+
+int launch_qmm_n_ws(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                    const void* biases, int64_t K, int gs, int bits, void* y, int y_dtype, void* workspace,
+                    size_t workspace_bytes, hipStream_t stream) {
+  if (y_dtype == dtype && workspace && aligned16(workspace) && prefer_frag_n(M, N, K, bits) &&
+      workspace_bytes >= qmm_frag_copy_bytes(K, N)) {
+    const int64_t tiles = ((M + BM - 1) / BM) * ((K + BN - 1) / BN);
+    TailPlan plan = plan_tail(M, K, N, 2, compute_units());
+    if (plan.splits > 1 && workspace_bytes < qmm_frag_copy_bytes(K, N) + tail_plane_bytes(M, K, plan))
+      plan = TailPlan{(int)tiles, 1};
+    float* planes = reinterpret_cast<float*>(static_cast<char*>(workspace) + qmm_frag_copy_bytes(K, N));
+    return launch_qmm_frag_n(x, dtype, M, N, wq, scales, biases, K, gs, bits, y, workspace, planes, plan.n_whole,
+                             plan.splits, stream);
+  }
+  return launch_qmm_n(x, dtype, M, N, wq, scales, biases, K, gs, bits, y, y_dtype, stream);
+}
+
 int launch_qmm(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,
                const void* biases, const void* bias, int64_t N, int gs, int bits, void* y, int y_dtype,
                void* workspace, size_t workspace_bytes, hipStream_t stream, LowRank low_rank, Epilogue epi) {

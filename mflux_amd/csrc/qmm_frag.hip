@@ -182,6 +182,61 @@ __global__ __launch_bounds__(256) void dequant_frag_stream_kernel(const uint32_t
   }
 }
 
+// The copy for the product with the weight NOT transposed (y[M, K] = x[M, N] @ dequantize(W[N, K]), the input
+// gradient of a quantized linear): the GEMM's output columns are then W's columns and its sum runs over W's
+// rows, so the copy holds W^T in fragment order -- blocks of 16 columns k x 64 rows n, a fragment the 8
+// consecutive n of one k.  A workgroup takes 64 rows x 256 columns: thread (rg, cg) = (t / 32, t % 32) loads the
+// 8 columns 8 cg .. of the 8 rows 8 rg .. (one word per row at 4 bits, two at 8: the 32 threads of a row
+// group read 128 or 256 contiguous bytes of each row), dequantises the 64 values and writes, per column, one
+// whole fragment into an LDS image of the 16 blocks; the image then leaves as 16-byte pieces in memory order.
+template <typename T, int GS, int BITS>
+__global__ __launch_bounds__(256) void dequant_frag_t_kernel(const uint32_t* __restrict__ wq,
+                                                             const uint16_t* __restrict__ scales,
+                                                             const uint16_t* __restrict__ biases,
+                                                             char* __restrict__ out, int N, int K, int tiles_k) {
+  __shared__ __attribute__((aligned(16))) char img[16 * kBlockBytes];
+  const int t = threadIdx.x;
+  const int rg = t >> 5, cg = t & 31;
+  const int st = blockIdx.x / tiles_k, tk = blockIdx.x - st * tiles_k;  // step of 64 rows, tile of 256 columns
+  const int steps = N / BK;
+  const int k0 = min(tk * 256 + 8 * cg, K - 8);  // columns past K (the last tile): the last eight again
+  constexpr int kWords = BITS / 4;               // words of 8 codes
+  uint32_t w[8][kWords];
+  float sc[8], bi[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int64_t n = (int64_t)st * BK + 8 * rg + i;
+#pragma unroll
+    for (int c = 0; c < kWords; ++c) w[i][c] = wq[(n * K + k0) * BITS / 32 + c];
+    sc[i] = T::to_f32(scales[n * (K / GS) + k0 / GS]);
+    bi[i] = T::to_f32(biases[n * (K / GS) + k0 / GS]);
+  }
+  // block cg / 2 of the tile, fragment (half, q, c16) = (rg % 2, rg / 2, 8 (cg % 2) + c)
+  char* dst = img + (cg >> 1) * kBlockBytes + 1024 * (rg & 1) + ((rg >> 1) * 16 + 8 * (cg & 1)) * 16;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t code = BITS == 4 ? (w[i][0] >> (4 * c)) & 0xfu : (w[i][c >> 2] >> (8 * (c & 3))) & 0xffu;
+      v[i] = __builtin_fmaf((float)code, sc[i], bi[i]);
+    }
+    *reinterpret_cast<u32x4*>(dst + 16 * c) =
+        u32x4{T::pack2(v[0], v[1]), T::pack2(v[2], v[3]), T::pack2(v[4], v[5]), T::pack2(v[6], v[7])};
+  }
+  __syncthreads();
+  // block b of the tile is block (16 tk + b) * steps + st of the copy; blocks past the copy's last are dropped
+  const int n_kb = (K + 15) / 16;
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    const int piece = p * 256 + t;  // 16-byte piece of the image
+    const int b = piece >> 7;
+    if (16 * tk + b < n_kb)
+      *reinterpret_cast<u32x4*>(out + ((int64_t)(16 * tk + b) * steps + st) * kBlockBytes + 16 * (piece & 127)) =
+          *reinterpret_cast<const u32x4*>(img + 16 * piece);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // 2. the GEMM.
 //
@@ -929,6 +984,46 @@ int launch_qmm_frag_gemm(const void* x, int dtype, int64_t M, int64_t K, const v
   if (dtype == MFQ_F16)
     return launch_gemm_typed<F16>(x, M, K, copy, bias, N, y, planes, n_whole, splits, stream, lr, epi);
   return MFQ_EDTYPE;
+}
+
+namespace {
+template <typename T, int GS>
+int launch_dequant_t_bits(const uint32_t* wq, const void* scales, const void* biases, int bits, void* out, int64_t N,
+                          int64_t K, hipStream_t stream) {
+  const int tiles_k = (int)((K + 255) / 256);
+  const dim3 grid((unsigned)((N / BK) * tiles_k));
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, wq, (const uint16_t*)scales, (const uint16_t*)biases,
+                       (char*)out, (int)N, (int)K, tiles_k);
+  };
+  if (bits == 4) go(dequant_frag_t_kernel<T, GS, 4>); else go(dequant_frag_t_kernel<T, GS, 8>);
+  return hipGetLastError() == hipSuccess ? MFQ_OK : MFQ_ELAUNCH;
+}
+template <typename T>
+int launch_dequant_t(const uint32_t* wq, const void* scales, const void* biases, int gs, int bits, void* out, int64_t N,
+                     int64_t K, hipStream_t stream) {
+  if (gs == 32) return launch_dequant_t_bits<T, 32>(wq, scales, biases, bits, out, N, K, stream);
+  if (gs == 64) return launch_dequant_t_bits<T, 64>(wq, scales, biases, bits, out, N, K, stream);
+  return launch_dequant_t_bits<T, 128>(wq, scales, biases, bits, out, N, K, stream);
+}
+}  // namespace
+
+// The two-kernel path for the weight NOT transposed: y[M, K] = x[M, N] @ dequantize(wq[N, K]).  The GEMM sees
+// K output columns and sums over N.  4 and 8 bits, 16-bit y of x's type, whole pairs of 64-row steps.
+bool qmm_frag_n_shape_ok(int64_t M, int64_t N, int64_t K, int bits) {
+  return (bits == 4 || bits == 8) && K % 8 == 0 && N * K < ((int64_t)1 << 31) && qmm_frag_shape_ok(M, K, N, bits);
+}
+
+int launch_qmm_frag_n(const void* x, int dtype, int64_t M, int64_t N, const uint32_t* wq, const void* scales,
+                      const void* biases, int64_t K, int gs, int bits, void* y, void* workspace, float* planes,
+                      int n_whole, int splits, hipStream_t stream) {
+  if (!qmm_frag_n_shape_ok(M, N, K, bits)) return MFQ_EUNSUPPORTED;
+  int rc = MFQ_EDTYPE;
+  if (dtype == MFQ_BF16) rc = launch_dequant_t<BF16>(wq, scales, biases, gs, bits, workspace, N, K, stream);
+  if (dtype == MFQ_F16) rc = launch_dequant_t<F16>(wq, scales, biases, gs, bits, workspace, N, K, stream);
+  if (rc) return rc;
+  return launch_qmm_frag_gemm(x, dtype, M, N, workspace, nullptr, K, y, planes, n_whole, splits, stream, LowRank(),
+                              Epilogue());
 }
 
 int launch_qmm_frag(const void* x, int dtype, int64_t M, int64_t K, const uint32_t* wq, const void* scales,

@@ -200,9 +200,14 @@ std::tuple<Tensor, bool> qmm_n(const Tensor& x, const Tensor& wq, const Tensor& 
   Tensor y = at::empty({M, K}, x.options().dtype(out_dtype));
   if (M == 0) return {y, true};
   const int sb = dtype_code(scales.scalar_type(), "scales");
-  const int rc = mfq_qmm_n(x.data_ptr(), sb, M, N, static_cast<const uint32_t*>(wq.data_ptr()), scales.data_ptr(),
-                           biases.data_ptr(), sb, K, (int)group_size, (int)bits, y.data_ptr(),
-                           dtype_code(out_dtype, "the output"), stream_of(x));
+  // the transposed 16-bit copy of the two-kernel path (and the planes of its K cut), where that is used
+  const size_t ws_bytes = mfq_qmm_n_workspace_bytes(M, N, K, (int)group_size, (int)bits);
+  Tensor ws;
+  if (ws_bytes) ws = at::empty({(int64_t)ws_bytes}, x.options().dtype(at::kByte));
+  const int rc = mfq_qmm_n_ws(x.data_ptr(), sb, M, N, static_cast<const uint32_t*>(wq.data_ptr()), scales.data_ptr(),
+                              biases.data_ptr(), sb, K, (int)group_size, (int)bits, y.data_ptr(),
+                              dtype_code(out_dtype, "the output"), ws_bytes ? ws.data_ptr() : nullptr, ws_bytes,
+                              stream_of(x));
   if (rc == MFQ_EUNSUPPORTED) return {y, false};
   check_status("mfq_qmm_n", rc);
   return {y, true};

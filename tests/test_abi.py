@@ -110,6 +110,16 @@ def test_argument_validation_needs_no_device():
     assert call_n(y=base + 8) == E["align"]
     assert call_n(bits=7) == E["bits"]
     assert call_n(N=12) == E["unsupported"]          # x rows are read in 16-byte pieces
+    nws = lib.mfq_qmm_n_ws                            # the same checks in front of the workspace form
+    assert nws(base, _lib.BF16, 4, 8, base, base, base, _lib.BF16, 100, 64, 4, base, _lib.BF16, None, 0, None) == E["shape"]
+    assert nws(base, _lib.F32, 4, 8, base, base, base, _lib.BF16, 128, 64, 4, base, _lib.BF16, None, 0, None) == E["dtype"]
+    nbytes = lib.mfq_qmm_n_workspace_bytes
+    assert nbytes(4608, 21504, 3072, 64, 4) >= 3072 * 21504 * 2    # the transposed 16-bit copy (and planes)
+    assert nbytes(4608, 21504, 3072, 64, 8) >= 3072 * 21504 * 2
+    assert nbytes(4608, 21504, 3072, 64, 5) == 0      # 3, 5 and 6 bits: the one-kernel form only
+    assert nbytes(512, 21504, 3072, 64, 4) == 0       # few rows of x: the one-kernel form
+    assert nbytes(4608, 200, 3072, 64, 4) == 0        # the reduction is not whole pairs of 64
+    assert nbytes(4608, 21504, 3000, 64, 4) == 0      # an error of the call itself: no workspace
 
     # the LoRA entry points: the rank comes in steps of 16 with both matrices present and aligned
     lr = lib.mfq_qmm_t_low_rank

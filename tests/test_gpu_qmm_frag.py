@@ -90,6 +90,80 @@ def test_two_kernel_path_scratch_copy_and_product(oracle, bits, gs, dtype, with_
     assert not torch.equal(y_fused, torch.zeros_like(y_fused))
 
 
+# The untransposed product (the input gradient) on the same GEMM: the copy is the TRANSPOSE of the dequantised
+# weight in fragment order.  10 x 13 tiles, the last column of tiles ragged; N (the reduction) of four, three and
+# five pairs of 64
+@pytest.mark.parametrize("bits,gs,dtype,N", [
+    (4, 64, "bf16", 512), (8, 64, "bf16", 512), (4, 32, "f16", 384), (8, 128, "f16", 640), (4, 128, "bf16", 640),
+    (8, 32, "bf16", 384)])
+def test_two_kernel_path_untransposed_copy_and_product(oracle, bits, gs, dtype, N):
+    from gpu_util import to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    M, K = 2400, {32: 3232, 64: 3264, 128: 3200}[gs]     # whole groups: the output width is a multiple of 32
+    k16 = (K + 15) // 16 * 16
+    need = lib.mfq_qmm_n_workspace_bytes(M, N, K, gs, bits)
+    assert need == k16 * N * 2, "the shape must take the two-kernel path, uncut"
+    g = o._from_f32(seeded(120 + bits + gs, 0, (M, N), 1.0), dt)
+    w = o._from_f32(seeded(120 + bits + gs, 1, (N, K), 0.02), dt)
+    wq, s, b = o.c_quantize(w, dt, gs, bits)
+    gd, wd, sd, bd = to_dev(g, dt), u32_to_dev(wq), to_dev(s, dt), to_dev(b, dt)
+    stream = torch.cuda.current_stream().cuda_stream
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    y = torch.empty(M, K, dtype=gd.dtype, device="cuda")
+    print(f"bits={bits} gs={gs} {dtype} M={M} N={N} K={K}", flush=True)
+    assert lib.mfq_qmm_n_ws(gd.data_ptr(), code, M, N, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), code, K, gs, bits,
+                            y.data_ptr(), code, ws.data_ptr(), need, stream) == 0
+    torch.cuda.synchronize()
+
+    # blocks of 16 output columns k x 64 n as [half][q][c16][8], value (q, half, e) = n 16 q + 8 half + e
+    copy = ws.view(torch.int16).view(k16 // 16, N // 64, 2, 4, 16, 8).permute(0, 4, 1, 3, 2, 5).reshape(k16, N)
+    got = copy.cpu().numpy().view(np.uint16)
+    w_hat = o.dequantize_exact(wq, s, b, dt, gs, bits)                     # [N, K] in float64, exact
+    want = o._from_f32(w_hat.astype(np.float32), dt).T                      # [K, N]
+    assert np.array_equal(got[:K], want)
+
+    ref = _to_f64(o, g, dt) @ w_hat
+    row_inf = np.abs(ref).max(axis=-1, keepdims=True)
+    err = np.abs(y.double().cpu().numpy() - ref) / row_inf
+    assert err.max() <= TOL, err.max()
+
+    # the one-kernel form of the same call (no workspace): same bound
+    y_one = torch.empty_like(y)
+    assert lib.mfq_qmm_n(gd.data_ptr(), code, M, N, wd.data_ptr(), sd.data_ptr(), bd.data_ptr(), code, K, gs, bits,
+                         y_one.data_ptr(), code, stream) == 0
+    torch.cuda.synchronize()
+    assert (np.abs(y_one.double().cpu().numpy() - ref) / row_inf).max() <= TOL
+
+
+def test_two_kernel_path_untransposed_one_hot_and_k_cut(oracle):
+    """One-hot rows of x pick rows of the dequantised weight, rounded once: bit
+    for bit.  And a shape whose tile sequence has a tail, cut along the
+    reduction into float32 planes (19 x 14 tiles = 266 on 256 compute units)."""
+    import mflux_amd
+    from gpu_util import raw, to_dev, u32_to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    for bits in (4, 8):
+        M, N, K = 4700, 1024, 3520
+        assert lib.mfq_qmm_n_workspace_bytes(M, N, K, 64, bits) > (K + 15) // 16 * 16 * N * 2 + 255, "planes too"
+        w = o.f32_to_bf16_bits(seeded(130 + bits, 1, (N, K), 0.02))
+        wq, s, b = o.c_quantize(w, o.BF16, 64, bits)
+        hot = (np.arange(M) * 5 + 3) % N
+        x = np.zeros((M, N), dtype=np.float32)
+        x[np.arange(M), hot] = 1.0
+        y = mflux_amd.quantized_matmul(to_dev(o.f32_to_bf16_bits(x), o.BF16), u32_to_dev(wq), to_dev(s, o.BF16),
+                                       to_dev(b, o.BF16), transpose=False, group_size=64, bits=bits)
+        expect = o.f32_to_bf16_bits(o.dequantize_exact(wq, s, b, o.BF16, 64, bits).astype(np.float32))[hot]
+        assert np.array_equal(raw(y), expect)
+
+
 def test_workspace_tells_the_path():
     """The workspace the library asks for tells which path a shape takes: the 16-bit
     copy (plus the planes of a K cut behind it) from 2048 activation rows on, the
