@@ -230,12 +230,32 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
   const int64_t wave_stride = (int64_t)gridDim.x * 4 * kWave;  // groups between a wavefront's iterations
   const Divisor by_bins(n_bins);
 
-  for (int64_t g0 = ((int64_t)blockIdx.x * 4 + wave) * kWave; g0 < n_groups; g0 += wave_stride) {
+  const int64_t g_first = ((int64_t)blockIdx.x * 4 + wave) * kWave;
+  auto store_group = [&](int64_t g, const uint32_t (&words)[kWords], float scale, float bias) __attribute__((always_inline)) {
+    if (g < n_groups) {
+      uint32_t* out = wq + g * kWords;  // 4 * kWords bytes per group: the widest store that stays aligned
+      if constexpr (kWords % 4 == 0) {
+#pragma unroll
+        for (int k = 0; k < kWords / 4; ++k)
+          reinterpret_cast<uint4*>(out)[k] = make_uint4(words[4 * k], words[4 * k + 1], words[4 * k + 2], words[4 * k + 3]);
+      } else if constexpr (kWords % 2 == 0) {
+#pragma unroll
+        for (int k = 0; k < kWords / 2; ++k) reinterpret_cast<uint2*>(out)[k] = make_uint2(words[2 * k], words[2 * k + 1]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < kWords; ++k) out[k] = words[k];
+      }
+      scales[g] = T::from_f32(scale);
+      biases[g] = T::from_f32(bias);
+    }
+  };
+  for (int64_t g0 = g_first; g0 < n_groups; g0 += wave_stride) {
     uint4 raw[kChunks];
+    // pieces past the end re-read the last one (no branch around a load): their groups are never stored
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
       const int64_t c = g0 * kChunks + j * kWave + lane;
-      raw[j] = c < n_chunks ? w16[c] : make_uint4(0, 0, 0, 0);
+      raw[j] = w16[c < n_chunks ? c : n_chunks - 1];
     }
 #pragma unroll
     for (int j = 0; j < kChunks; ++j) {
@@ -274,15 +294,32 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
     uint32_t words[kWords];
     uint64_t stream = 0;
     int stream_bits = 0, n_words = 0;
-    auto pack = [&](int, const uint32_t (&code)[8]) __attribute__((always_inline)) {
+    // code[e]: integral values in [0, n_bins].  4 and 8 bits go to bytes with one instruction each (even and odd
+    // codes of a 4-bit word in two registers, joined by one shift-or); the other widths through the bit stream.
+    auto pack = [&](int i, const float (&code)[8]) __attribute__((always_inline)) {
+      if constexpr (BITS == 8 || BITS == 4) {
+        uint32_t lo = 0, hi = 0;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        stream |= (uint64_t)code[e] << stream_bits;
-        stream_bits += BITS;
-        if (stream_bits >= 32) {
-          words[n_words++] = (uint32_t)stream;
-          stream >>= 32;
-          stream_bits -= 32;
+        for (int e = 0; e < 4; ++e) {
+          lo = __builtin_amdgcn_cvt_pk_u8_f32(code[BITS == 8 ? e : 2 * e], e, lo);
+          hi = __builtin_amdgcn_cvt_pk_u8_f32(code[BITS == 8 ? 4 + e : 2 * e + 1], e, hi);
+        }
+        if constexpr (BITS == 8) {
+          words[2 * i] = lo;
+          words[2 * i + 1] = hi;
+        } else {
+          words[i] = lo | (hi << 4);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          stream |= (uint64_t)(uint32_t)code[e] << stream_bits;
+          stream_bits += BITS;
+          if (stream_bits >= 32) {
+            words[n_words++] = (uint32_t)stream;
+            stream >>= 32;
+            stream_bits -= 32;
+          }
         }
       }
     };
@@ -298,11 +335,11 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
       const Divisor by_scale(scale);
 #pragma unroll
       for (int i = 0; i < kChunks; ++i) {
-        uint32_t code[8];
+        float code[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float q = rintf(by_scale.divide(element(i, e) - bias));
-          code[e] = (uint32_t)__builtin_amdgcn_fmed3f(q, 0.0f, n_bins);
+          code[e] = __builtin_amdgcn_fmed3f(q, 0.0f, n_bins);
         }
         pack(i, code);
       }
@@ -317,34 +354,18 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
       }
 #pragma unroll
       for (int i = 0; i < kChunks; ++i) {
-        uint32_t code[8];
+        float code[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           float q = rintf((element(i, e) - bias) / scale);
           q = (q < 0.0f) ? 0.0f : q;
           q = (n_bins < q) ? n_bins : q;
-          code[e] = (uint32_t)q;
+          code[e] = (float)(uint32_t)q;  // (a NaN becomes code 0 here)
         }
         pack(i, code);
       }
     }
-    const int64_t g = g0 + lane;
-    if (g < n_groups) {
-      uint32_t* out = wq + g * kWords;  // 4 * kWords bytes per group: the widest store that stays aligned
-      if constexpr (kWords % 4 == 0) {
-#pragma unroll
-        for (int k = 0; k < kWords / 4; ++k)
-          reinterpret_cast<uint4*>(out)[k] = make_uint4(words[4 * k], words[4 * k + 1], words[4 * k + 2], words[4 * k + 3]);
-      } else if constexpr (kWords % 2 == 0) {
-#pragma unroll
-        for (int k = 0; k < kWords / 2; ++k) reinterpret_cast<uint2*>(out)[k] = make_uint2(words[2 * k], words[2 * k + 1]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < kWords; ++k) out[k] = words[k];
-      }
-      scales[g] = T::from_f32(scale);
-      biases[g] = T::from_f32(bias);
-    }
+    store_group(g0 + lane, words, scale, bias);
   }
 }
 
@@ -520,9 +541,14 @@ int quantize_bits(const void* w, int64_t n_chunks, int bits, uint32_t* wq, void*
   using S = typename T::storage;
   if constexpr (sizeof(S) == 2) {
     const int64_t n_groups = n_chunks / (GS / 8);
-    const int64_t blocks = (n_groups + 4 * kWave - 1) / (4 * kWave);  // four wavefronts of 64 groups each
-    const int64_t cap = 256 * 4;  // resident at once on 256 CUs; wavefronts loop over the rest
-    const int grid = (int)(blocks < cap ? blocks : cap);
+    // A wavefront takes 64 groups per trip.  At most 256 * 4 workgroups of four wavefronts are resident at
+    // once on 256 CUs; beyond that every wavefront makes the same number of trips (fewer wavefronts rather than
+    // a last round that only some of them run).
+    const int64_t wave_trips = (n_groups + kWave - 1) / kWave;
+    const int64_t cap_waves = 256 * 4 * 4;
+    const int64_t trips = (wave_trips + cap_waves - 1) / cap_waves;
+    const int64_t waves = (wave_trips + trips - 1) / trips;
+    const int grid = (int)((waves + 3) / 4);
     auto launch = [&](auto kernel) {
       hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales, (S*)biases, n_groups);
     };
