@@ -381,6 +381,20 @@ int mfq_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, cons
                             const void* shift, int64_t rows_per_vector, float eps, void* y, void* stream);
 
 /*
+ * t[M, rank] = x[M, K] @ A[K, rank]: the down-projection of the adapters,
+ * mx.matmul(x, lora_A) of src/mflux/models/common/lora/layer/linear_lora_layer.py:50-53
+ * for all adapters of a layer at once, A = [lora_A_1 | lora_A_2 | ...] (zero
+ * columns up to a multiple of 16).  A is packed once per adapter set, so it is
+ * handed over in the order the matrix instruction consumes, af
+ * [rank/16][K/32][4][16][8]: af[f][s][q][c][e] = A[32 s + 8 q + e][16 f + c].
+ * x, af and t are of the 16-bit type dtype; the sums are float32, rounded
+ * once.  rank % 16 == 0, rank <= 1024, K % 32 == 0.  t is the first operand of
+ * mfq_qmm_t_low_rank and mfq_low_rank_add.
+ */
+int mfq_low_rank_down(const void* x, const void* af, int dtype, int64_t M, int64_t K, int64_t rank, void* t,
+                      void* stream);
+
+/*
  * y[M, N] += t[M, rank] @ bs[N, rank]^T in float32, rounded to y_dtype (dtype
  * or MFQ_F32): the same adapters (see mfq_qmm_t_low_rank for t and bs) behind
  * a product that did not come from mfq_qmm_t_low_rank, e.g. one of the matvec

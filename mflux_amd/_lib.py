@@ -43,6 +43,7 @@ SIGNATURES = {
                                   _I64, _PTR, _INT, _PTR, ctypes.c_size_t, _PTR]),
     "mfq_qmv_silu": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _PTR, _INT, _PTR, _I64, _INT, _INT, _PTR, _INT, _PTR]),
     "mfq_layer_norm_modulate": (_INT, [_PTR, _INT, _I64, _I64, _PTR, _PTR, _I64, ctypes.c_float, _PTR, _PTR]),
+    "mfq_low_rank_down": (_INT, [_PTR, _PTR, _INT, _I64, _I64, _I64, _PTR, _PTR]),
     "mfq_low_rank_add": (_INT, [_PTR, _PTR, _INT, _I64, _I64, _I64, _PTR, _INT, _PTR]),
 }
 

@@ -318,6 +318,17 @@ int mfq_layer_norm_modulate(const void* x, int dtype, int64_t M, int64_t K, cons
                                          (hipStream_t)stream);
 }
 
+int mfq_low_rank_down(const void* x, const void* at, int dtype, int64_t M, int64_t K, int64_t rank, void* t,
+                      void* stream) {
+  if (!is16(dtype)) return MFQ_EDTYPE;
+  if (M <= 0 || K <= 0 || M > INT32_MAX || K > INT32_MAX || K % 32) return MFQ_ESHAPE;
+  if (rank <= 0 || rank > 1024 || rank % 16) return MFQ_ESHAPE;
+  if (M * K >= (int64_t)1 << 40) return MFQ_ESHAPE;
+  if (!x || !at || !t) return MFQ_ENULL;
+  if (!mfq::aligned16(x) || !mfq::aligned16(at) || !mfq::aligned16(t)) return MFQ_EALIGN;
+  return mfq::launch_low_rank_down(x, dtype, M, K, at, rank, t, (hipStream_t)stream);
+}
+
 int mfq_low_rank_add(const void* t, const void* bs, int dtype, int64_t M, int64_t N, int64_t rank, void* y, int y_dtype,
                      void* stream) {
   if (!is16(dtype)) return MFQ_EDTYPE;

@@ -359,6 +359,9 @@ int launch_qmm_epilogue(const void* x, int dtype, int64_t M, int64_t K, const ui
                         void* workspace, size_t workspace_bytes, hipStream_t stream, Epilogue epi);
 // y[M, N] += t @ bs^T, rounded to y's type (dtype: the type of t, bs and a 16-bit y)
 int launch_low_rank_add(int dtype, LowRank low_rank, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t stream);
+// t[M, R] = x[M, K] @ A[K, R], A in fragment order ([R/16][K/32][4][16][8]); 16-bit type `dtype`; R % 16 == 0, K % 32 == 0
+int launch_low_rank_down(const void* x, int dtype, int64_t M, int64_t K, const void* at, int64_t R, void* t,
+                         hipStream_t stream);
 // what a caller should bring (the K split's planes, or the scratch copy of the two-kernel path where that is
 // preferred) and what the call cannot do without (the planes only)
 size_t qmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int gs, int bits);

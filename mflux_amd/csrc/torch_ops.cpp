@@ -257,6 +257,20 @@ std::tuple<Tensor, bool> layer_norm_modulate(const Tensor& x, const c10::optiona
   return {y, true};
 }
 
+// t = x @ A, A in the fragment order of mfq_low_rank_down ([R/16, K/32, 4, 16, 8])
+Tensor low_rank_down(const Tensor& x, const Tensor& af) {
+  TORCH_CHECK(x.dim() == 2 && af.dim() == 5 && x.is_contiguous() && af.is_contiguous() && af.size(2) == 4 &&
+                  af.size(3) == 16 && af.size(4) == 8 && x.size(1) == 32 * af.size(1) &&
+                  x.scalar_type() == af.scalar_type(),
+              "mfq::low_rank_down: x [M, K], af [R/16, K/32, 4, 16, 8], contiguous, of one 16-bit type");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  const int64_t R = 16 * af.size(0);
+  Tensor t = at::empty({x.size(0), R}, x.options());
+  check_status("mfq_low_rank_down", mfq_low_rank_down(x.data_ptr(), af.data_ptr(), dtype_code(x.scalar_type(), "x"),
+                                                      x.size(0), x.size(1), R, t.data_ptr(), stream_of(x)));
+  return t;
+}
+
 // y += t @ bs^T in place
 void low_rank_add_(Tensor& y, const Tensor& t, const Tensor& bs) {
   TORCH_CHECK(y.dim() == 2 && t.dim() == 2 && bs.dim() == 2 && y.is_contiguous() && t.is_contiguous() &&
@@ -281,6 +295,7 @@ TORCH_LIBRARY(mfq, m) {
   m.def("qmv_silu(Tensor x, Tensor wq, Tensor scales, Tensor biases, Tensor? bias, int group_size, int bits) -> (Tensor, bool)");
   m.def("layer_norm_modulate(Tensor x, Tensor? scale, Tensor? shift, float eps) -> (Tensor, bool)");
   m.def("low_rank_add_(Tensor(a!) y, Tensor t, Tensor bs) -> ()");
+  m.def("low_rank_down(Tensor x, Tensor af) -> Tensor");
 }
 
 TORCH_LIBRARY_IMPL(mfq, CUDA, m) {  // the HIP backend answers to torch's CUDA dispatch key
@@ -293,4 +308,5 @@ TORCH_LIBRARY_IMPL(mfq, CUDA, m) {  // the HIP backend answers to torch's CUDA d
   m.impl("qmv_silu", qmv_silu);
   m.impl("layer_norm_modulate", layer_norm_modulate);
   m.impl("low_rank_add_", low_rank_add_);
+  m.impl("low_rank_down", low_rank_down);
 }

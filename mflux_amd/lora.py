@@ -21,7 +21,7 @@ import math
 
 import torch
 
-from . import core
+from . import _lib, core
 from .nn import Linear, QuantizedLinear
 
 _RANK_STEP = 16  # the kernels take the low rank in steps of 16
@@ -93,13 +93,27 @@ def pack_adapters(loras: list[LoRALinear], dtype: torch.dtype) -> tuple[torch.Te
     return a_cat.contiguous(), bs.contiguous()
 
 
+_DOWN_KERNEL_MAX_K = 4096
+
+
+def down_fragments(a_cat: torch.Tensor) -> torch.Tensor:
+    """``a_cat [K, R]`` (``K % 32 == 0``, ``R % 16 == 0``) in the order the
+    down-projection kernel's matrix instruction consumes it:
+    ``[R/16, K/32, 4, 16, 8]`` with ``af[f, s, q, c, e] = a_cat[32 s + 8 q + e, 16 f + c]``."""
+    K, R = a_cat.shape
+    if K % 32 or R % 16:
+        raise ValueError(f"[down_fragments] a_cat must be [K, R] with K % 32 == 0 and R % 16 == 0, got {tuple(a_cat.shape)}")
+    return a_cat.reshape(K // 32, 4, 8, R // 16, 16).permute(3, 0, 1, 4, 2).contiguous()
+
+
 def _packed_for(owner: torch.nn.Module, loras: list[LoRALinear], dtype: torch.dtype):
     # rebuilt when an adapter's tensors are replaced or written in place, or a scale changes
     key = (dtype,) + tuple((id(lora), lora.lora_A.data_ptr(), lora.lora_A._version, lora.lora_B.data_ptr(),
                             lora.lora_B._version, float(lora.scale)) for lora in loras)
     cache = owner.__dict__.get("_packed_adapters")
     if cache is None or cache[0] != key:
-        cache = (key, pack_adapters(loras, dtype))
+        a_cat, bs = pack_adapters(loras, dtype)
+        cache = (key, (a_cat, down_fragments(a_cat) if a_cat.shape[0] <= _DOWN_KERNEL_MAX_K else None, bs))
         owner.__dict__["_packed_adapters"] = cache
     return cache[1]
 
@@ -115,9 +129,17 @@ def _forward(owner: torch.nn.Module, base: torch.nn.Module, loras: list[LoRALine
     if not fused:
         return _composed(base, loras, x)
     compute = base.scales.dtype
-    a_cat, bs = _packed_for(owner, loras, compute)
-    # the down-projection is a plain skinny GEMM: the BLAS library's split-K kernels run it at memory speed
-    t = torch.matmul(x.to(compute), a_cat)
+    a_cat, af, bs = _packed_for(owner, loras, compute)
+    # t = x @ [lora_A_1 | lora_A_2 | ...], float32 sums rounded once.  Rows of up to 4096 elements (the hidden
+    # sizes of the transformer blocks): one read of x in csrc/lora.hip, on a par with or ahead of the BLAS
+    # library.  Longer rows (the MLP down-projections, K = 10240 .. 15360): the library's skinny split-K GEMM,
+    # which is 1.2-1.7x faster there (the kernel re-reads a fragment of lora_A per 16 rows of x, which costs
+    # the vector memory path as much as the x it meets).
+    K = x.shape[-1]
+    if K <= _DOWN_KERNEL_MAX_K:
+        t = _lib.ops().low_rank_down(x.to(compute).reshape(-1, K).contiguous(), af).reshape(*x.shape[:-1], bs.shape[1])
+    else:
+        t = torch.matmul(x.to(compute), a_cat)
     return core.quantized_matmul(x, base.weight, base.scales, base.biases, transpose=True, group_size=base.group_size,
                                  bits=base.bits, mode=base.mode, bias=base.bias, low_rank=(t, bs))
 

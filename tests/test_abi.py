@@ -20,7 +20,7 @@ def declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("mfq_version", "mfq_strerror", "mfq_quantize_affine", "mfq_dequantize_affine", "mfq_dequantize_rows",
-                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add",
+                 "mfq_qmm_t", "mfq_qmm_t_ws", "mfq_qmm_t_workspace_bytes", "mfq_qmm_t_low_rank", "mfq_low_rank_add", "mfq_low_rank_down",
                  "mfq_qmm_t_prepare", "mfq_qmm_t_prepared", "mfq_qmm_t_prepared_bytes", "mfq_qmm_t_prepared_workspace_bytes",
                  "mfq_qmv_silu"):
         assert must in names
@@ -143,6 +143,13 @@ def test_argument_validation_needs_no_device():
     assert add(base, base, _lib.BF16, 4, 8, 24, base, _lib.BF16, None) == E["shape"]
     assert add(base, None, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["null"]
     assert add(base + 8, base, _lib.BF16, 4, 8, 16, base, _lib.BF16, None) == E["align"]
+    down = lib.mfq_low_rank_down                      # t [M, rank] = x [M, K] @ at [rank, K]^T
+    assert down(base, base, _lib.F32, 4, 64, 16, base, None) == E["dtype"]
+    assert down(base, base, _lib.BF16, 4, 48, 16, base, None) == E["shape"]     # K in steps of 32
+    assert down(base, base, _lib.BF16, 4, 64, 24, base, None) == E["shape"]     # the rank in steps of 16
+    assert down(base, base, _lib.BF16, 0, 64, 16, base, None) == E["shape"]
+    assert down(base, None, _lib.BF16, 4, 64, 16, base, None) == E["null"]
+    assert down(base, base + 8, _lib.BF16, 4, 64, 16, base, None) == E["align"]
     # the two halves of the large-M call apart: which shapes have a prepared copy, and the checks of both calls
     nbytes = lib.mfq_qmm_t_prepared_bytes
     assert nbytes(3072, 3072, 4) == 3072 * 3072 * 2 and nbytes(3208, 512, 8) == 3216 * 512 * 2
@@ -205,7 +212,7 @@ def test_torch_ops_are_registered_and_refuse_cpu_tensors():
     from mflux_amd import _lib
 
     ops = _lib.ops()
-    for name in ("quantize_affine", "dequantize_affine", "dequantize_rows", "qmm_t", "qmv_silu", "low_rank_add_"):
+    for name in ("quantize_affine", "dequantize_affine", "dequantize_rows", "qmm_t", "qmv_silu", "low_rank_add_", "low_rank_down"):
         assert hasattr(ops, name), name
     with pytest.raises(NotImplementedError, match="CPU"):
         ops.quantize_affine(torch.zeros(2, 64, dtype=torch.bfloat16), 64, 4)

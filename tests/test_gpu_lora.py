@@ -139,6 +139,51 @@ def test_low_rank_update_is_exact_on_integers(oracle):
     assert torch.equal(y.double(), ref)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("M,K,R", [
+    (4608, 3072, 16),      # the single-block linear1 with one rank-16 adapter: six steps of 32 k per wavefront
+    (100, 15360, 48),      # ragged rows, three fragments of columns, thirty steps per wavefront
+    (17, 96, 80),          # fewer steps (3) than wavefronts (16); two column blocks (64 + 16)
+    (1, 32, 16),           # one row, one step
+    (333, 1056, 128),      # 33 steps: the wavefronts' shares are uneven (3, 3, ..., 0)
+])
+def test_down_projection_vs_f64(oracle, dtype, M, K, R):
+    """t = x @ A through the C ABI (at = A^T, [R, K]): float32 sums of exact products, rounded once:
+    within one rounding of the float64 value (2^-8 relative for bfloat16, 2^-11
+    for float16, of the row's largest |t|, plus the float32 summation error)."""
+    from gpu_util import raw, to_dev
+    from mflux_amd import _lib
+
+    o = oracle
+    lib = _lib.load()
+    dt = o.BF16 if dtype == "bf16" else o.F16
+    code = _lib.BF16 if dtype == "bf16" else _lib.F16
+    x = o._from_f32(seeded(140 + R, 0, (M, K), 1.0), dt)
+    at = o._from_f32(seeded(140 + R, 1, (R, K), 1.0 / np.sqrt(K)), dt)
+    # A = at^T in the order the kernel wants it: af[f, s, q, c, e] = A[32 s + 8 q + e, 16 f + c]
+    f_, s_, q_, c_, e_ = np.indices((R // 16, K // 32, 4, 16, 8))
+    af = np.ascontiguousarray(at.T[32 * s_ + 8 * q_ + e_, 16 * f_ + c_])
+    xd, ad = to_dev(x, dt), to_dev(af.reshape(-1, 8), dt)
+    guard = torch.full((M + 2, R), 7.0, device="cuda", dtype=xd.dtype)
+    t = guard[1:M + 1]
+    print(f"{dtype} M={M} K={K} R={R}", flush=True)
+    assert lib.mfq_low_rank_down(xd.data_ptr(), ad.data_ptr(), code, M, K, R, t.data_ptr(),
+                                 torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    ref = o._to_f32(x, dt).astype(np.float64) @ o._to_f32(at, dt).astype(np.float64).T
+    err = np.abs(t.double().cpu().numpy() - ref) / np.abs(ref).max(axis=1, keepdims=True)
+    assert err.max() <= (2.0 ** -8 if dtype == "bf16" else 2.0 ** -11) * 1.05, err.max()
+    assert bool((guard[0] == 7.0).all()) and bool((guard[M + 1] == 7.0).all())
+    # one-hot rows pick columns of at, bit for bit
+    hot = (np.arange(M) * 7 + 3) % K
+    xh = np.zeros((M, K), dtype=np.float32)
+    xh[np.arange(M), hot] = 1.0
+    th = torch.empty(M, R, device="cuda", dtype=xd.dtype)
+    assert lib.mfq_low_rank_down(to_dev(o._from_f32(xh, dt), dt).data_ptr(), ad.data_ptr(), code, M, K, R,
+                                 th.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    assert np.array_equal(raw(th), at[:, hot].T)
+
+
 def test_low_rank_argument_checks():
     import mflux_amd
 

@@ -455,3 +455,22 @@ def test_update_module_writes_into_shared_storage():
     lin = torch.nn.ModuleDict({"l": qnn.Linear(64, 8, bias=False)})
     W.update_module(lin, {"l": {"weight": torch.zeros(8, 8, dtype=torch.int32).view(torch.uint32)}})
     assert lin["l"].weight.dtype == torch.uint32 and tuple(lin["l"].weight.shape) == (8, 8)
+
+
+def test_down_projection_fragment_order():
+    """The stacked lora_A as the down-projection kernel reads it: fragment f, step
+    s, lane 16 q + c holds a_cat[32 s + 8 q .. + 7, 16 f + c]."""
+    import numpy as np
+    import torch
+
+    from mflux_amd.lora import down_fragments
+
+    a = torch.arange(96 * 48, dtype=torch.float32).reshape(96, 48)
+    af = down_fragments(a)
+    assert tuple(af.shape) == (3, 3, 4, 16, 8) and af.is_contiguous()
+    f, s, q, c, e = np.indices(af.shape)
+    assert np.array_equal(af.numpy(), a.numpy()[32 * s + 8 * q + e, 16 * f + c])
+    with pytest.raises(ValueError):
+        down_fragments(torch.zeros(40, 16))
+    with pytest.raises(ValueError):
+        down_fragments(torch.zeros(64, 8))
