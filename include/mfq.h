@@ -235,8 +235,9 @@ int mfq_qmm_n_ws(const void* x, int x_dtype, int64_t M, int64_t N, const uint32_
  * cut into ranges that run on different compute units, each range accumulates
  * into its own float32 plane of the workspace, and a second kernel adds the
  * planes, rounds and applies the bias (same two roundings as the fused
- * epilogue).  Large calls -- 4 or 8 bits, 16-bit y, K a multiple of 128, at
- * least 2048 activation rows (where it starts to pay), e.g. the single-stream
+ * epilogue).  Large calls -- 16-bit y, K a multiple of 128, at least 2048
+ * activation rows at 4 or 8 bits and 1024 at 3, 5 or 6 (where it starts to
+ * pay), e.g. the single-stream
  * linears of FLUX.1 at M = 4608 -- use the workspace first for a 16-bit copy of
  * the dequantised weights (round_up(N, 16) * K * 2 bytes rounded up to 256,
  * written once per call in the order the matrix instructions consume it) and
@@ -265,14 +266,13 @@ int mfq_qmm_t_ws(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_
  * 16-bit copy of the dequantised weights that mfq_qmm_t_ws makes per call --
  * one rounding of fma(code, scale, bias) to sb_dtype, in the order the matrix
  * instructions consume it, mfq_qmm_t_prepared_bytes(N, K, bits) bytes (2 per
- * weight; 0: no such copy for this shape: bits other than 4 or 8, K not a
+ * weight; 0: no such copy for this shape: K not a
  * multiple of 128 or below 256, N not a multiple of 8, or more than 2 GiB) --
  * into a buffer the caller keeps, and mfq_qmm_t_prepared multiplies x
  * [M, K] of the same 16-bit type with it into y [M, N] of that type (+ bias):
  * bit-identical to what mfq_qmm_t_ws gives on its two-kernel path, for any M,
  * at 2 bytes per weight of memory held instead of bits / 8 -- on FLUX.1's
- * single-block linears at M = 4608 the copy is 7 % of the call.  The copy can
- * also be made on another stream while the previous layer's product runs.
+ * single-block linears at M = 4608 the copy is 7 % of the call.
  * `workspace` (optional, 16-byte aligned, mfq_qmm_t_prepared_workspace_bytes)
  * takes the float32 planes of a K cut of a short last round of tiles; without
  * it the tiles run whole.  MFQ_EUNSUPPORTED for shapes without a copy.
@@ -324,9 +324,10 @@ int mfq_qmm_t_static(const void* x, int x_dtype, int64_t M, int64_t K, const uin
  * mfq_qmm_t does for M <= 4.  Arguments as for mfq_qmm_t.
  * MFQ_EUNSUPPORTED when no fused kernel takes the shape (bits other than 4
  * and 8; M = 1 with rows of more than 6 KiB of 8-bit or 3 KiB of 4-bit codes;
- * M = 2..4 outside what the four-rows kernel takes: K > 4096, N not a multiple
- * of 4, rows that are not 1, 2, 3, 4, 6, 8, 12 or 16 times 256 bytes; M > 4):
- * apply the activation separately and call mfq_qmm_t.
+ * M = 2..4 outside what the eight-rows kernels (K = 1024, 2048, 3072 or 4096,
+ * group size 64, N a multiple of 8) and the four-rows kernel (K <= 4096, N a
+ * multiple of 4, rows of 1, 2, 3, 4, 6, 8, 12 or 16 times 256 bytes) take;
+ * M > 4): apply the activation separately and call mfq_qmm_t.
  */
 int mfq_qmv_silu(const void* x, int x_dtype, int64_t M, int64_t K, const uint32_t* wq,
                  const void* scales, const void* biases, int sb_dtype, const void* bias, int64_t N,
