@@ -303,6 +303,13 @@ def baseline_configs(torch, mflux_amd, dev, quick=False):
     flops = 2.0 * 4096 * 3072 * 3072
     out["config1_flux_to_q_m4096_w4"] = {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
                                          "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    # the same layer with its 16-bit copy kept (QuantizedLinear.prepare(): 2 bytes per weight held, the call is
+    # the GEMM alone): a variant beside the configuration's figure, not instead of it
+    lin.prepare()
+    ms = timed(lambda: lin(x), 10, 50)
+    out["config1_flux_to_q_m4096_w4"]["with_kept_copy"] = {
+        "us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
+        "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
     del lin, x
 
     # -- 4: Z-Image block, M = 4352, hidden 3840, W8, no bias: q, k, v, out, w1, w3, w2
@@ -328,6 +335,11 @@ def baseline_configs(torch, mflux_amd, dev, quick=False):
         ms = timed(fn, 5, 20)
         res[key] = {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
                     "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    held = sum(int(layer.prepare()) * 2 * layer.output_dims * layer.input_dims for layer in (q, k, v, o, w1, w3, w2))
+    ms = timed(separate, 5, 20)
+    res["seven_calls_with_kept_copies"] = {"us": round(ms * 1e3, 1), "tflops": round(flops / ms / 1e9, 1),
+                                           "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                                           "copies_held_gb": round(held / 1e9, 2)}
     out["config4_zimage_block_m4352_w8"] = res
     del q, k, v, o, w1, w3, w2, qkv, gate_up, x, xh
 
@@ -396,6 +408,17 @@ def baseline_configs(torch, mflux_amd, dev, quick=False):
         ms = timed(fn, 1, 2 if not quick else 1)
         res[key] = {"ms_per_step": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
                     "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    # the image stream's linears with their 16-bit copies kept (13.6 GB more for the 60 blocks; the text stream's
+    # 256 rows do not use one)
+    held = 0
+    for streams in blocks:
+        for key in ("qkv", "out", "mlp_in", "mlp_out"):
+            layer = streams[0][key]
+            held += int(layer.prepare()) * 2 * layer.output_dims * layer.input_dims
+    ms = timed(step_two_streams, 1, 2 if not quick else 1)
+    res["qkv_as_one_two_hip_streams_and_kept_copies"] = {
+        "ms_per_step": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
+        "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "copies_held_gb": round(held / 1e9, 2)}
     out["config5_qwen_image_step_w4"] = res
     del blocks
     torch.cuda.empty_cache()
