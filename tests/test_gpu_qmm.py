@@ -801,6 +801,72 @@ def test_shape_sweep_against_oracle(oracle, case):
     _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs), row_floor=0.02 * x_norm)
 
 
+# The borders that the row count and the tile count draw between the large-M paths: 1024 rows (3, 5 and 6 bits
+# move from the 128-column-tile kernel to the two-kernel path; the untransposed product likewise at 4 and 8 bits),
+# 2048 rows (4 and 8 bits move from the fused kernel to the two-kernel path), each with just enough 256 x 256 tiles
+# for those paths to be taken; and the shapes on either side of what the eight-rows matvecs take.
+_LARGE_BORDERS = [
+    # M, K, N, bits, gs, transpose
+    (1023, 512, 8456, 5, 64, True), (1024, 512, 8456, 5, 64, True), (1025, 384, 8712, 3, 32, True),
+    (1024, 640, 8448, 6, 128, True), (2047, 512, 3848, 4, 64, True), (2048, 512, 3848, 4, 64, True),
+    (2049, 384, 3848, 8, 32, True), (2048, 256, 4104, 8, 128, True), (1500, 512, 8456, 4, 64, True),
+    (2048, 512, 3840, 6, 64, True), (1024, 512, 8440, 3, 64, True),
+    # untransposed: x [M, N] @ dequant(w [N, K]) -> [M, K]
+    (1023, 8448, 512, 4, 64, False), (1024, 8448, 512, 4, 64, False), (1025, 8512, 384, 8, 32, False),
+    (2049, 3872, 512, 4, 32, False), (2048, 3840, 640, 8, 128, False), (2048, 3840, 576, 4, 64, False),
+    (1024, 8448, 512, 5, 64, False),
+]
+
+
+@pytest.mark.parametrize("case", _LARGE_BORDERS, ids=lambda c: "M%d-K%d-N%d-w%d-g%d-%s" % c)
+def test_large_m_borders_against_oracle(oracle, case):
+    import mflux_amd
+    from gpu_util import to_dev, u32_to_dev
+
+    o = oracle
+    M, K, N, bits, gs, transpose = case
+    print(case, flush=True)
+    if transpose:
+        args = _case(o, 700 + M % 97 + bits, M, K, N, bits, gs=gs, with_bias=bool(M % 2))
+        _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs))
+        return
+    w = o.f32_to_bf16_bits(seeded(800 + bits, 1, (N, K), 0.02))
+    wq, s, b = o.c_quantize(w, o.BF16, gs, bits)
+    g = o.f32_to_bf16_bits(seeded(800 + bits, 5, (M, N), 1.0))
+    ref = o.bf16_bits_to_f32(g).astype(np.float64) @ o.dequantize_exact(wq, s, b, o.BF16, gs, bits)
+    y = mflux_amd.quantized_matmul(to_dev(g, o.BF16), u32_to_dev(wq), to_dev(s, o.BF16), to_dev(b, o.BF16),
+                                   transpose=False, group_size=gs, bits=bits)
+    assert tuple(y.shape) == (M, K)
+    _assert_close(y, ref)
+
+
+def _matvec_border_cases():
+    rng = np.random.default_rng(20241125)
+    cases = []
+    for i in range(24):
+        M = int(rng.choice([1, 2, 3, 4, 5]))
+        K = int(rng.choice([1024, 2048, 3072, 4096, 5120, 1088, 960]))
+        N = int(rng.choice([8, 72, 100, 2312, 20, 9224]))
+        bits = int(rng.choice([4, 8]))
+        gs = int(rng.choice([64, 64, 64, 32, 128]))
+        if K % gs:
+            K = K // gs * gs
+        cases.append((i, M, K, N, bits, gs))
+    return cases
+
+
+@pytest.mark.parametrize("case", _matvec_border_cases(), ids=lambda c: "case%d-M%d-K%d-N%d-w%d-g%d" % c)
+def test_matvec_borders_against_oracle(oracle, case):
+    """Shapes on both sides of what the eight-rows matvecs take (K in steps of 1024
+    up to 4096, groups of 64, N a multiple of 8, one to four rows): whichever
+    kernel takes the call, the product holds the tolerance."""
+    o = oracle
+    i, M, K, N, bits, gs = case
+    args = _case(o, 900 + i, M, K, N, bits, gs=gs, with_bias=bool(i % 2))
+    x_norm = np.linalg.norm(o.bf16_bits_to_f32(args[0]).astype(np.float64), axis=-1, keepdims=True)
+    _assert_close(_run(o, *args, bits, gs), _ref(o, *args, bits, gs), row_floor=0.02 * x_norm)
+
+
 def test_torch_ops_and_ctypes_routes_agree_bit_for_bit(oracle):
     """The two ways into libmfq -- torch.ops.mfq (what mflux_amd.core uses) and the
     C ABI through ctypes -- run the same kernels on the same stream: quantize,
