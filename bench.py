@@ -419,8 +419,29 @@ def baseline_configs(torch, mflux_amd, dev, quick=False):
     res["qkv_as_one_two_hip_streams_and_kept_copies"] = {
         "ms_per_step": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
         "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4), "copies_held_gb": round(held / 1e9, 2)}
+    # ... and the 120 modulation linears of the step (they all take the same silu(temb)) as one matvec over their
+    # stacked rows at the start of the step (nn.concat_quantized(share_storage=True): the layers become views)
+    mods = qnn.concat_quantized([s_["mod"] for streams in blocks for s_ in streams], share_storage=True)
+
+    def step_two_streams_one_modulation():
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            qnn.silu_linear(mods, temb)
+            for streams in blocks:
+                s_ = streams[1]
+                s_["qkv"](xt), s_["out"](xt), s_["mlp_in"](xt), s_["mlp_out"](xth)
+        for streams in blocks:
+            s_ = streams[0]
+            s_["qkv"](xi), s_["out"](xi), s_["mlp_in"](xi), s_["mlp_out"](xih)
+        main.wait_stream(side)
+
+    ms = timed(step_two_streams_one_modulation, 1, 2 if not quick else 1)
+    res["qkv_as_one_two_hip_streams_kept_copies_and_one_modulation_call"] = {
+        "ms_per_step": round(ms, 2), "tflops": round(flops / ms / 1e9, 1),
+        "frac_mfma": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
     out["config5_qwen_image_step_w4"] = res
-    del blocks
+    del blocks, mods
     torch.cuda.empty_cache()
     return out
 
