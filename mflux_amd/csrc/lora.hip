@@ -108,8 +108,9 @@ int launch(LowRank lr, int64_t M, int64_t N, void* y, int y_dtype, hipStream_t s
 //
 // x is read once (2 M K bytes: the kernel is bound by that read, and the whole of it is only a few times what
 // must be in flight to cover the memory latency), so the work is cut for memory parallelism, not for the matrix
-// cores: a workgroup of 8 wavefronts owns 16 rows of x, wavefront w a contiguous eighth of K, and a wavefront
-// requests a whole trip (four pairs of 32-k steps: 8 KiB of x) before it uses any of it.
+// cores: a workgroup of 8 wavefronts owns 16 rows of x, the trips (four pairs of 32-k steps: 512 bytes of each row,
+// 8 KiB of x) are dealt to its wavefronts in turn, so that the workgroup reads one 4 KiB window of every row at a
+// time, and a wavefront requests a whole trip before it uses any of it and the next one while it computes.
 //   - the vector memory path takes about as long per cache line touched as per 128 bytes moved, so every load
 //     covers whole lines: x goes row-segment-wise (8 lanes = one 128-byte line of a row) through a private LDS
 //     region of the wavefront (no barrier), XOR-swizzled so that the fragment reads are conflict free;
@@ -137,8 +138,9 @@ __global__ __launch_bounds__(kDownWaves* kWave, 2) void low_rank_down_kernel(con
   char* stage = lds + wave * kDownStage;
 
   const int steps = K / 32, pairs = (steps + 1) / 2;
-  const int per_wave = (pairs + kDownWaves - 1) / kDownWaves;
-  const int p_begin = min(wave * per_wave, pairs), p_end = min(p_begin + per_wave, pairs);
+  // trips are dealt round-robin: trip t of wavefront w is pairs (t * 8 + w) * 4 .. + 3, so that at any time the
+  // workgroup reads one window of 4 KiB per row (16 pages in flight instead of 128)
+  const int p_begin = wave * kDownPairs, p_end = pairs, p_stride = kDownWaves * kDownPairs;
   // staging: piece h (0, 1) of a pair is rows 8 h + lane / 8, 16-byte column lane % 8 of the pair's 128 bytes;
   // in LDS the column is XORed with row % 8.  A pair's second step may lie past K (K % 64 == 32): its columns
   // re-read the first step's and are not used.
@@ -169,13 +171,13 @@ __global__ __launch_bounds__(kDownWaves* kWave, 2) void low_rank_down_kernel(con
   };
   u32x4 xr[kDownPairs][2];
   if (p_begin < p_end) request(xr, p_begin);
-  for (int p0 = p_begin; p0 < p_end; p0 += kDownPairs) {
+  for (int p0 = p_begin; p0 < p_end; p0 += p_stride) {
 #pragma unroll
     for (int u = 0; u < kDownPairs; ++u)
 #pragma unroll
       for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4*>(stage + u * 2048 + sput[h]) = xr[u][h];
     // the next trip's x is on its way while this one meets its fragments of A
-    if (p0 + kDownPairs < p_end) request(xr, p0 + kDownPairs);
+    if (p0 + p_stride < p_end) request(xr, p0 + p_stride);
     // (the region is private to the wavefront, whose LDS operations complete in order: no barrier)
 #pragma unroll
     for (int u = 0; u < kDownPairs; ++u) {

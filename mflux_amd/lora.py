@@ -133,8 +133,7 @@ def _forward(owner: torch.nn.Module, base: torch.nn.Module, loras: list[LoRALine
     # t = x @ [lora_A_1 | lora_A_2 | ...], float32 sums rounded once.  Rows of up to 4096 elements (the hidden
     # sizes of the transformer blocks): one read of x in csrc/lora.hip, on a par with or ahead of the BLAS
     # library.  Longer rows (the MLP down-projections, K = 10240 .. 15360): the library's skinny split-K GEMM,
-    # which is 1.2-1.7x faster there (the kernel re-reads a fragment of lora_A per 16 rows of x, which costs
-    # the vector memory path as much as the x it meets).
+    # which is 1.2-1.6x faster there (the kernel streams such rows from memory at 3.5 TB/s only).
     K = x.shape[-1]
     if K <= _DOWN_KERNEL_MAX_K:
         t = _lib.ops().low_rank_down(x.to(compute).reshape(-1, K).contiguous(), af).reshape(*x.shape[:-1], bs.shape[1])
