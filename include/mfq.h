@@ -24,8 +24,7 @@
  *     word i / (32/bits); for 3, 5 and 6 bits it is MLX's 3- and 5-byte packs
  *     laid end to end.  scales and biases hold one value per `group_size`
  *     consecutive elements of a row.
- *   - bits: 3, 4, 5, 6, 8 everywhere (quantize of 3, 5, 6 bits takes 16-bit
- *     inputs only).
+ *   - bits: 3, 4, 5, 6, 8 everywhere.
  */
 #ifndef MFQ_H
 #define MFQ_H

@@ -76,9 +76,6 @@ def quantize(w: torch.Tensor, group_size: int = 64, bits: int = 4, mode: str = "
             "[quantize] The last dimension of the matrix needs to be divisible by the quantization "
             f"group size {group_size}. However the provided matrix has shape {tuple(w.shape)}"
         )
-    if bits not in MATMUL_KERNEL_BITS and w.dtype == torch.float32:
-        raise NotImplementedError(f"[quantize] {bits}-bit quantization of float32 input is not implemented in "
-                                  "this build; cast to bfloat16 or float16")
     _require_hip("quantize", w, "w")
     lead = tuple(w.shape[:-1])
     wq, scales, biases = _lib.ops().quantize_affine(w.reshape(-1, K).contiguous(), group_size, bits)

@@ -389,6 +389,65 @@ __global__ __launch_bounds__(256) void quantize_group_per_lane_kernel(const uint
   }
 }
 
+// float32 input at 3, 5 and 6 bits (a checkpoint kept in float32 and mflux's -q 3/5/6,
+// src/mflux/cli/defaults/defaults.py:63): one lane per group, which it reads twice -- for its limits, then for
+// its codes, the second time out of the caches -- so that no more than eight values live in registers at a
+// time; the arithmetic is the scalar algorithm statement by statement (exact divisions), the codes leave as the
+// group's little-endian bit stream, scales and biases as float32.  A pass over weights this wide is rare (the
+// models' weights arrive in 16 bits), so nothing here is tuned: each lane's loads are its own 4 GS bytes.
+template <int GS, int BITS>
+__global__ __launch_bounds__(256) void quantize_f32_stream_kernel(const float* __restrict__ w,
+                                                                  uint32_t* __restrict__ wq,
+                                                                  float* __restrict__ scales,
+                                                                  float* __restrict__ biases, int64_t n_groups) {
+  constexpr int kWords = GS * BITS / 32;
+  constexpr float n_bins = (float)((1 << BITS) - 1);
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n_groups; g += stride) {
+    const float4* src = reinterpret_cast<const float4*>(w + g * GS);
+    float w_min = src[0].x, w_max = w_min;
+#pragma unroll 4
+    for (int i = 0; i < GS / 4; ++i) {
+      const float4 v = src[i];
+      w_min = fminf(fminf(fminf(w_min, v.x), fminf(v.y, v.z)), v.w);
+      w_max = fmaxf(fmaxf(fmaxf(w_max, v.x), fmaxf(v.y, v.z)), v.w);
+    }
+    const bool mask = fabsf(w_min) > fabsf(w_max);
+    const float edge = mask ? w_min : w_max;
+    float scale = (w_max - w_min) / n_bins, bias = 0.0f;
+    scale = (scale < kEps) ? kEps : scale;
+    scale = mask ? scale : -scale;
+    const float q0 = rintf(edge / scale);
+    if (q0 != 0.0f) {
+      scale = edge / q0;
+      bias = edge;
+    }
+    uint32_t* out = wq + g * kWords;
+    uint64_t stream = 0;
+    int stream_bits = 0, n_words = 0;
+#pragma unroll
+    for (int i = 0; i < GS / 4; ++i) {
+      const float4 v = src[i];
+      const float x[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float q = rintf((x[e] - bias) / scale);
+        q = (q < 0.0f) ? 0.0f : q;
+        q = (n_bins < q) ? n_bins : q;
+        stream |= (uint64_t)(uint32_t)q << stream_bits;  // (a NaN becomes code 0 here)
+        stream_bits += BITS;
+        if (stream_bits >= 32) {
+          out[n_words++] = (uint32_t)stream;
+          stream >>= 32;
+          stream_bits -= 32;
+        }
+      }
+    }
+    scales[g] = scale;
+    biases[g] = bias;
+  }
+}
+
 // code * scale + bias as mx.dequantize evaluates it: an element-wise multiply and
 // an element-wise add on arrays of the output type, so the product is rounded
 // to that type before the bias is added and the sum is rounded again by the
@@ -580,9 +639,18 @@ int quantize_bits(const void* w, int64_t n_chunks, int bits, uint32_t* wq, void*
       default: launch(quantize_group_per_lane_kernel<T, GS, 8>); break;
     }
   } else {
-    if (bits != 4 && bits != 8) return MFQ_EUNSUPPORTED;  // float32 input: 4 and 8 bits only
     const int grid = grid_for(n_chunks, kUnroll);
-    if (bits == 4) {
+    if (bits == 3 || bits == 5 || bits == 6) {
+      const int64_t n_groups = n_chunks / (GS / 8);
+      const int g = grid_for(n_groups, 1);
+      auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(g), dim3(256), 0, stream, (const float*)w, wq, (float*)scales, (float*)biases,
+                           n_groups);
+      };
+      if (bits == 3) launch(quantize_f32_stream_kernel<GS, 3>);
+      if (bits == 5) launch(quantize_f32_stream_kernel<GS, 5>);
+      if (bits == 6) launch(quantize_f32_stream_kernel<GS, 6>);
+    } else if (bits == 4) {
       hipLaunchKernelGGL((quantize_kernel<T, GS, 4>), dim3(grid), dim3(256), 0, stream, (const S*)w, wq, (S*)scales,
                          (S*)biases, n_chunks);
     } else {

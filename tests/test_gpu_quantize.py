@@ -242,3 +242,37 @@ def test_odd_bit_widths_full_size_weight(oracle):
     got = mflux_amd.quantize(to_dev(w, o.BF16), group_size=64, bits=5)
     for e, g in zip(exp, got):
         assert np.array_equal(raw(g), e)
+
+
+@pytest.mark.parametrize("bits", [3, 5, 6])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_odd_bit_widths_float32_input_bit_exact(oracle, bits, gs):
+    """float32 weights at 3, 5 and 6 bits: packed words and the float32 scales and
+    biases equal the oracle's on random, adversarial (ties, equal groups, tiny and
+    huge ranges, denormals) and exponent-sweeping groups; dequantize returns
+    the float32 product and sum of the same codes."""
+    import mflux_amd
+    from gpu_util import raw, to_dev, u32_to_dev
+
+    o = oracle
+    rows, K = 96, 1024
+    rng = np.random.default_rng(500 + 10 * bits + gs)
+    rnd = seeded(9, bits * 1000 + gs + 11, (rows, K), 0.02)
+    adv = _adversarial_groups(o, rows * K // gs, gs, seed=bits + gs + 3).reshape(rows, K)
+    sweep = (rng.standard_normal((rows * K // gs, gs), dtype=np.float32)
+             * np.exp2(rng.integers(-80, 60, size=(rows * K // gs, 1)).astype(np.float32))).reshape(rows, K)
+    for name, f32 in (("random", rnd), ("adversarial", adv), ("sweep", sweep)):
+        f32 = np.ascontiguousarray(f32, dtype=np.float32)
+        exp = o.c_quantize(f32, o.F32, gs, bits)
+        got = mflux_amd.quantize(to_dev(f32, o.F32), group_size=gs, bits=bits)
+        for what, e, g in zip(("wq", "scales", "biases"), exp, got):
+            assert tuple(g.shape) == e.shape, (name, what)
+            bad = np.flatnonzero(raw(g).reshape(-1) != e.reshape(-1))
+            assert bad.size == 0, f"{name}/{what}: {bad.size} mismatches, first at {bad[:4]}"
+        assert got[1].dtype == torch.float32 and got[2].dtype == torch.float32
+    wq, s, b = exp
+    with np.errstate(all="ignore"):
+        exp32 = o.c_dequantize(wq, s, b, o.F32, gs, bits)
+    d32 = mflux_amd.dequantize(u32_to_dev(wq), to_dev(s, o.F32), to_dev(b, o.F32), group_size=gs, bits=bits)
+    ok = np.isfinite(exp32)
+    assert d32.dtype == torch.float32 and np.array_equal(raw(d32)[ok], exp32[ok])
