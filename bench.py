@@ -707,6 +707,25 @@ def main():
                                                  "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
                                                  "bytes": nbytes}
         del picks, wq_all, s_all, b_all, bias_all
+        # the two modulation linears of ONE joint block (norm1 and norm1_context take the same text_embeddings,
+        # src/mflux/models/flux/model/flux_transformer/joint_transformer_block.py:29-38) as one call, pairs of
+        # weights in rotation: the smallest stack a block offers
+        pairs = [tuple(torch.cat([bufs[(2 * i) % n_buf][j], bufs[(2 * i + 1) % n_buf][j]]) for j in range(3))
+                 for i in range(n_buf // 2)]
+        bias_pair = bias.repeat(2)
+        state = {"i": 0}
+
+        def pair_call():
+            wqg, sg, bg = pairs[state["i"] % len(pairs)]
+            state["i"] += 1
+            mflux_amd.silu_quantized_matmul(temb16, wqg, sg, bg, group_size=GS, bits=bits_g, bias=bias_pair)
+
+        ms = graph_ms(pair_call, 4 * len(pairs), 10, torch)
+        nbytes = qmm_bytes(1, Kg, 2 * Ng, bits_g, bias=True)
+        res["M1_2_linears_of_a_block_one_call"] = {"us": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                                                   "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                                                   "bytes": nbytes}
+        del pairs, bias_pair
         res["M1_with_silu"] = {"fused_us": round(graph_ms(fused_call, 4 * n_buf, 10, torch) * 1e3, 2),
                                "separate_us": round(graph_ms(separate_call, 4 * n_buf, 10, torch) * 1e3, 2)}
         temb16 = seeded_bf16(torch, dev, 2, 0, (4, Kg), 1.0)  # the same for a batch of four
